@@ -17,7 +17,7 @@ extern "C" {
 #endif
 
 #define JL_API __attribute__((visibility("default")))
-#define JL_VERSION 110
+#define JL_VERSION 120
 #define JL_OK 0
 #define JL_E_INVALID (-1)
 #define JL_E_LAUNCH (-3)
@@ -37,6 +37,25 @@ JL_API int jl_embed_scale(const void *embed, int dtype, const int64_t *ids, int6
 JL_API int jl_add_rmsnorm(float *x, const void *y, int y_dtype, int32_t y_count, const float *x0, const void *w, float eps,
                           void *out, int dtype, int64_t N, int32_t W, void *stream);
 
+/* Residual update from several scaled addends, then up to two RMS norms of the SAME updated row with float weights stored around
+ * `w_offset` — the layer whose mixer and feed-forward both read one stream and are added in one sum:
+ *   x[n, c] += sum_a scale_a[c] * sum_{s < count_a} y_a[(n * count_a + s), c]        (at most 3 addends; scale null = 1)
+ *   out1[n] = x[n] / sqrt(mean(x[n]^2) + eps) * (w_offset + w1);   out2 likewise with w2   (out1 / out2 / w1 / w2 may be null)
+ * x float in place; y_a of its own dtype; out1 / out2 of `dtype`. */
+typedef struct { const void *y; int32_t dtype; int32_t count; const float *scale; } jl_addend;
+JL_API int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n_addends, const float *w1, const float *w2, float w_offset,
+                               float eps, void *out1, void *out2, int dtype, int64_t N, int32_t W, void *stream);
+
+/* Gated activation of a feed-forward whose gate and linear branch are column ranges of one product z [N, ld] (F columns each at
+ * g_col / u_col):   out[n, c] = act(g) * lin(u) * sigmoid(row_gate[n * rg_ld])        (row_gate null: no row gate)
+ *   JL_ACT_GELU_TANH:      act(g) = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), lin(u) = u
+ *   JL_ACT_CLAMPED_SWISH:  g' = min(g, limit), u' = clamp(u, -limit, limit); act = g' sigmoid(alpha g'), lin = u' + shift
+ * z, row_gate and out [N, F] of `dtype`; the arithmetic is float. */
+#define JL_ACT_GELU_TANH 0
+#define JL_ACT_CLAMPED_SWISH 1
+JL_API int jl_gated_act(const void *z, int dtype, int64_t N, int64_t ld, int32_t g_col, int32_t u_col, int32_t F, int32_t kind, float limit,
+                        float alpha, float shift, const void *row_gate, int64_t rg_ld, void *out, void *stream);
+
 /* Whole-projection query / key norm + cache append.  proj [N, ld] holds q (H*D columns at q_col), k (G*D at k_col) and v (G*Dv at
  * v_col).  q_out [N, H*D] = rms_norm(q) * wq over ALL H*D columns at once; the key is normalised the same way over G*D with wk and
  * stored at k_cache[slot[n]] ([pool tokens, G*D]); v is stored as it is at v_cache[slot[n]] ([pool tokens, G*Dv]).  slot < 0 skips
@@ -50,6 +69,9 @@ JL_API int jl_qk_norm_append(const void *proj, int dtype, int64_t N, int64_t ld,
  *   s_g(i, j) = q_g(i) . k_c(g)(j) * scale + rel[lut[min(i - j, lut_len - 1)], g]          (c(g) = g / (H / G))
  *   p_g(i, .) = softmax over the visible j;   w_h(i, j) = sum_g talk[h, g] p_g(i, j)  (talk null: w = p)
  *   out_h(i) = (sum_j w_h(i, j) v_c(h)(j)) * sigmoid(gate_h(i))                             (gate null: no gate)
+ * With `sink` (float [H], may be null) the softmax's denominator of head g holds one more term exp(sink[g]): a key without a value,
+ * neither scaled nor biased, counted once, so the weights of a row sum to less than one.  `gate` is read element by element
+ * ([N, H*Dv], rows gate_ld apart) or, with gate_heads != 0, one number per head ([N, H], rows gate_ld apart).
  * tiles [n_tiles, 4] int32 = {b, first query position, count (<= TQ), first row}: consecutive rows of one request;
  * block_tables [*, bt_stride] int32 pages of request b in order; a key j lives at token page * page_size + j % page_size of the
  * pool.  window <= 0 means no window (plain causal).  rel [rows, H] float and lut int32 may be null (no bias). */
@@ -65,6 +87,8 @@ typedef struct {
     int64_t k_ld, v_ld;           /* row stride of k_cache / v_cache in elements (0: G*D / Gv*Dv).  v_cache may point into k_cache.    */
     int32_t Gv;                   /* value heads (0: G).  G % Gv == 0; key head c reads value head c % Gv (score maps share values)   */
     int32_t out_dtype;            /* dtype of `out` when it differs from `dtype`: JL_OUT_F32 = float outputs from bfloat16 inputs     */
+    const float *sink;            /* float [H] or null: one more term exp(sink[g]) in head g's softmax denominator                    */
+    int32_t gate_heads;           /* != 0: `gate` holds one number per head ([N, H]) instead of one per output element                */
 } jl_attn_args;
 #define JL_OUT_SAME 0
 #define JL_OUT_F32 2
@@ -74,11 +98,11 @@ JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
  * they do not fit */
 JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld);
 
-/* The same attention without bias, head mixing and gate, in ONE sweep over the keys on the matrix cores, for heads in groups that
+/* The same attention without bias and head mixing (sink and gate as above), in ONE sweep over the keys on the matrix cores, for heads in groups that
  * share a key head (H / G query heads per key head c, value head c % Gv): bfloat16, D % 8 == 0 up to 640, Dv % 32 == 0 up to 512,
  * row strides % 4 == 0.  v_cache == k_cache (with G = 1, Dv <= D): the values are the first Dv columns of the key rows — the pool
  * of latent attention — and are not loaded a second time.  Of jl_attn_args it reads q, k_cache, v_cache, k_ld, v_ld, out, out_dtype,
- * block_tables, bt_stride, tiles, n_tiles, page_size, H, G, Gv, D, Dv, window, scale, dtype, splits, scratch and TQ, which must be
+ * block_tables, bt_stride, tiles, n_tiles, page_size, H, G, Gv, D, Dv, window, scale, dtype, sink, gate, gate_ld, gate_heads, splits, scratch and TQ, which must be
  * what jl_attn_sweep_tile_rows returns (0: sizes not taken).  splits in 2 .. 64: the keys of every tile are shared out over that
  * many workgroups and joined by a second launch; `scratch` then holds jl_attn_sweep_scratch_floats floats. */
 JL_API int jl_attn_sweep(const jl_attn_args *a, void *stream);
@@ -107,17 +131,19 @@ JL_API int jl_causal_conv(const float *x, const void *w, int dtype, const int32_
                           int64_t N, int32_t W, int32_t taps, void *out, void *stream);
 JL_API int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t B, float *tail, int32_t W, int32_t taps, void *stream);
 
-/* Per-head query / key norm for attention with M score maps per head, query temperature, cache append.  proj [N, ld] holds q
- * (H heads x M maps x D at q_col, head by head), k (G x M x D at k_col) and v (G x Dv at v_col).  Every D-vector is RMS-normalised on
- * its own and multiplied by wq / wk [D]; the query is further multiplied by 1 + t_coef * ln(floor((p + 1) / t_every) + 1), p = pos[n]
- * (t_coef 0: no temperature).  Queries and keys are written MAP-major — q_out [N, M, H, D], k_cache[slot[n]] = [M, G, D] — so that
+/* Per-head query / key stage for attention with M score maps per head: rotation, norm, query temperature, cache append.  proj
+ * [N, ld] holds q (H heads x M maps x D at q_col, head by head), k (G x M x D at k_col) and v (G x Dv at v_col).  With rot_dims > 0
+ * every D-vector is first rotated by its position p = pos[n]: of its first rot_dims dimensions, i and i + rot_dims/2 form a pair
+ * (u, v) -> (u cos a - v sin a, v cos a + u sin a), a from the cos / sin tables [positions, rot_dims/2] float; the rest pass unchanged.
+ * Every D-vector is then RMS-normalised on its own and multiplied by wq / wk [D] (null: no weight); the query is further multiplied by
+ * 1 + t_coef * ln(floor((p + 1) / t_every) + 1) (t_coef 0: no temperature).  Queries and keys are written MAP-major — q_out [N, M, H, D], k_cache[slot[n]] = [M, G, D] — so that
  * query row m*H + h reads key row (m*H + h) / (H/G) = m*G + h/(H/G) and value head (m*G + g) % G: one attention launch with M*H query
  * heads, M*G key heads and G value heads computes all maps.  With maps_apart != 0 the queries are written [M, N, H, D] instead: one
  * launch per map, each over its own G*D columns of the key rows.  v goes to v_cache[slot[n]] as it is. */
 JL_API int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t H,
                                int32_t G, int32_t M, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, float t_coef,
                                int32_t t_every, const int32_t *pos, void *q_out, int32_t maps_apart, void *k_cache, void *v_cache,
-                               const int64_t *slot, void *stream);
+                               const int64_t *slot, int32_t rot_dims, const float *cos_t, const float *sin_t, void *stream);
 
 /* Differential combination of two score maps' outputs a1, a2 (float, rows of H*Dv values `ld` floats apart):
  * o = a1 - lambda * a2;  out[n, h] = o / sqrt(mean(o^2) + eps) * out_scale over the head's Dv values; out [N, H*Dv] of `dtype`. */
@@ -166,10 +192,15 @@ JL_API int jl_retention(const void *proj, int dtype, int64_t ld, int32_t q_col, 
 JL_API int jl_retention_join(const int32_t *req, int32_t B, const int32_t *chunk_len, int32_t H, int32_t D, int32_t Dv,
                              const float *decay, float *state, float *scratch, void *stream);
 
-/* Router of a mixture of experts: s = sigmoid(logits) (float [N, E]); the `top` experts with the largest s + correction are
- * chosen (ties: lowest index); ids [N, top] int32, weights [N, top] float = s * scale (not renormalised). */
+/* Router of a mixture of experts over float logits [N, E]; ids [N, top] int32, weights [N, top] float.
+ *   JL_ROUTE_SIGMOID:        s = sigmoid(logits); the `top` experts with the largest s + correction are chosen (ties: lowest
+ *                            index); weights = s * scale (not renormalised).
+ *   JL_ROUTE_SOFTMAX_RENORM: s = softmax(logits) over all experts; the `top` largest are chosen (ties: lowest index); weights =
+ *                            s / (sum of the chosen s + renorm_eps) * scale.  `correction` is not read. */
+#define JL_ROUTE_SIGMOID 0
+#define JL_ROUTE_SOFTMAX_RENORM 1
 JL_API int jl_moe_route(const float *logits, const float *correction, int64_t N, int32_t E, int32_t top, float scale, int32_t *ids,
-                        float *weights, void *stream);
+                        float *weights, int32_t kind, float renorm_eps, void *stream);
 
 /* Rows (token, choice) grouped by expert.  perm [N*top]: sorted row -> flat index n*top + s; offsets [E+1]; tile_expert /
  * tile_row0 [max_tiles] (max_tiles >= N*top/tile_rows + E): row tiles of at most tile_rows rows of one expert, unused entries -1. */
@@ -179,7 +210,10 @@ JL_API int jl_moe_tile_rows(void);
 
 /* Grouped product over the sorted rows: C[r, :] = X[in(r), :] . W[e(r)]^T with W [E, n_out, K].
  *   mode 0 (up):   in(r) = perm[r] / top;  out[r, :] = relu(C)^2, stored in `dtype` ([N*top, n_out], sorted order)
- *   mode 1 (down): in(r) = r;              out[perm[r], :] = C * weights[perm[r]], stored as float ([N*top, n_out]) */
+ *   mode 1 (down): in(r) = r;              out[perm[r], :] = C * weights[perm[r]], stored as float ([N*top, n_out])
+ *   mode JL_MOE_UP_PLAIN: as mode 0 without the activation (out[r, :] = C): a gated unit stacks its gate and linear branch in W and
+ *                  applies jl_gated_act to the result */
+#define JL_MOE_UP_PLAIN 2
 JL_API int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mode, int32_t K, int32_t n_out, int32_t top,
                        const int32_t *perm, const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0,
                        int32_t max_tiles, const float *weights, void *out, void *stream);

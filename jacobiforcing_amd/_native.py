@@ -232,6 +232,9 @@ def raise_state_error(code: int, what: str, aux: int = 0):
 # ---- libjf_layers.so (include/jf_layers.h): layer kernels of the models whose forward is not stock PyTorch ----------------------------
 JL_F32, JL_BF16 = 0, 1
 JL_OUT_SAME, JL_OUT_F32 = 0, 2
+JL_ACT_GELU_TANH, JL_ACT_CLAMPED_SWISH = 0, 1
+JL_ROUTE_SIGMOID, JL_ROUTE_SOFTMAX_RENORM = 0, 1
+JL_MOE_UP_RELU2, JL_MOE_DOWN, JL_MOE_UP_PLAIN = 0, 1, 2
 
 
 class AttnArgs(C.Structure):
@@ -241,7 +244,12 @@ class AttnArgs(C.Structure):
                 ("bt_stride", _i32), ("n_tiles", _i32), ("lut_len", _i32), ("page_size", _i32), ("H", _i32), ("G", _i32), ("D", _i32),
                 ("Dv", _i32), ("window", _i32), ("keep_first", _i32), ("TQ", _i32), ("dtype", _i32), ("scale", _f32),
                 ("splits", _i32), ("n_rows", _i32), ("scratch", _vp), ("q_pack", _vp), ("k_ld", _i64), ("v_ld", _i64), ("Gv", _i32),
-                ("out_dtype", _i32)]
+                ("out_dtype", _i32), ("sink", _vp), ("gate_heads", _i32)]
+
+
+class Addend(C.Structure):
+    """jl_addend (include/jf_layers.h)."""
+    _fields_ = [("y", _vp), ("dtype", _i32), ("count", _i32), ("scale", _vp)]
 
 
 _LAYER_SIGNATURES = {
@@ -261,7 +269,9 @@ _LAYER_SIGNATURES = {
     "jl_causal_conv": (C.c_int, [_vp, _vp, C.c_int, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp]),
     "jl_causal_conv_carry": (C.c_int, [_vp, _vp, _i32, _vp, _i32, _i32, _vp]),
     "jl_head_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _f32, _i32,
-                                      _vp, _vp, _i32, _vp, _vp, _vp, _vp]),
+                                      _vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
+    "jl_scaled_add_norms": (C.c_int, [_vp, C.POINTER(Addend), _i32, _vp, _vp, _f32, _f32, _vp, _vp, C.c_int, _i64, _i32, _vp]),
+    "jl_gated_act": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _vp, _i64, _vp, _vp]),
     "jl_diff_combine": (C.c_int, [_vp, _vp, _i64, _i64, _i32, _i32, _f32, _f32, _f32, _vp, C.c_int, _vp]),
     "jl_latent_prep": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _vp, _vp,
                                  _vp, _vp]),
@@ -270,7 +280,7 @@ _LAYER_SIGNATURES = {
     "jl_retention": (C.c_int, [_vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _f32,
                                _vp, _vp, _i32, _vp]),
     "jl_retention_join": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp]),
-    "jl_moe_route": (C.c_int, [_vp, _vp, _i64, _i32, _i32, _f32, _vp, _vp, _vp]),
+    "jl_moe_route": (C.c_int, [_vp, _vp, _i64, _i32, _i32, _f32, _vp, _vp, _i32, _f32, _vp]),
     "jl_moe_group": (C.c_int, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp]),
     "jl_moe_tile_rows": (C.c_int, []),
     "jl_moe_gemm": (C.c_int, [_vp, _vp, C.c_int, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp]),

@@ -113,7 +113,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
     const T *vc = (const T *)a.v_cache;
 
     for (int e = tid; e < cnt * H * D; e += ATT_THREADS) Qs[e] = ld_f(q + (int64_t)row0 * H * D + e);
-    for (int e = tid; e < H * TQ; e += ATT_THREADS) { mx[e] = -INFINITY; sm[e] = 0.f; }
+    // a sink is a key without a value: every row starts from its score with a sum of one
+    for (int e = tid; e < H * TQ; e += ATT_THREADS) { mx[e] = a.sink ? a.sink[e / TQ] : -INFINITY; sm[e] = a.sink ? 1.f : 0.f; }
     if (a.talk) for (int e = tid; e < H * H; e += ATT_THREADS) talk[e] = a.talk[e];
 
     float acc[ACC];
@@ -207,7 +208,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
         if (e < cnt * H * Dv) {
             const int ii = e / (H * Dv), r = e - ii * (H * Dv);
             float v = acc[x];
-            if (gate) v *= 1.0f / (1.0f + expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + r)));
+            if (gate) v *= 1.0f / (1.0f + expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + (a.gate_heads ? r / Dv : r))));
             if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[(int64_t)(row0 + ii) * (H * Dv) + r] = v;
             else st_f(out + (int64_t)(row0 + ii) * (H * Dv) + r, v);
         }
@@ -359,6 +360,17 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
     for (int x = 0; x < HPW; ++x)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { m_run[x][r] = -INFINITY; l_run[x][r] = 0.f; }
+    if (a.sink && split == 0 && l32 == 0) {                         // the sink enters every row's statistics once: first share, one lane per row
+#pragma unroll
+        for (int x = 0; x < HPW; ++x) {
+            const int g = wave * HPW + x;
+            if (g < H) {
+                const float sk = a.sink[g];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) { m_run[x][r] = sk; l_run[x][r] = 1.f; }
+            }
+        }
+    }
 
     // fetch one tile ahead when a thread's share of a tile fits the registers set aside for it (one head per wavefront only: with
     // two the accumulators leave no room)
@@ -571,7 +583,7 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
                 if (ii >= cnt) continue;
                 const int col = h * Dv + 32 * t + l32;
                 float v = acc[x][t][r];
-                if (gate) v *= 1.0f / (1.0f + __expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + col)));
+                if (gate) v *= 1.0f / (1.0f + __expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + (a.gate_heads ? h : col))));
                 if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[(int64_t)(row0 + ii) * (H * Dv) + col] = v;
                 else st_f(out + (int64_t)(row0 + ii) * (H * Dv) + col, v);
             }
@@ -596,14 +608,15 @@ __global__ __launch_bounds__(256) void attn_pack_q_kernel(const bf16_t *__restri
 
 // out = gate * the sum of the splits' shares, in split order
 __global__ __launch_bounds__(256) void attn_join_kernel(const float *__restrict__ po, int S, int64_t total, int width,
-                                                         const bf16_t *__restrict__ gate, int64_t gate_ld, bf16_t *__restrict__ out, int out_f32) {
+                                                         const bf16_t *__restrict__ gate, int64_t gate_ld, int gate_every,
+                                                         bf16_t *__restrict__ out, int out_f32) {
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= total) return;
     float v = 0.f;
     for (int sp = 0; sp < S; ++sp) v += po[(int64_t)sp * total + e];
     if (gate) {
         const int64_t row = e / width;
-        v *= 1.0f / (1.0f + __expf(-ld_f(gate + row * gate_ld + (e - row * width))));
+        v *= 1.0f / (1.0f + __expf(-ld_f(gate + row * gate_ld + (e - row * width) / gate_every)));      // gate_every = Dv: one gate per head
     }
     if (out_f32) ((float *)out)[e] = v;
     else st_f(out + e, v);
@@ -633,7 +646,8 @@ template <int HPW, int NDV> static int am_launch(const jl_attn_args &a, hipStrea
     kern<<<grid, 64 * waves, lds, st>>>(a, AM_PV);
     const int64_t total = (int64_t)a.n_rows * a.H * a.Dv;
     attn_join_kernel<<<dim3((unsigned)((total + 255) / 256)), 256, 0, st>>>(a.scratch + (int64_t)a.n_tiles * a.splits * a.H * AM_T * 2, a.splits, total,
-                                                                          a.H * a.Dv, (const bf16_t *)a.gate, a.gate_ld, (bf16_t *)a.out, a.out_dtype == JL_OUT_F32);
+                                                                          a.H * a.Dv, (const bf16_t *)a.gate, a.gate_ld, a.gate_heads ? a.Dv : 1, (bf16_t *)a.out,
+                                                                          a.out_dtype == JL_OUT_F32);
     return jl_check_launch("attn_mfma_kernel (split keys)");
 }
 

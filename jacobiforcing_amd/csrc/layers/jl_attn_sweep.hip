@@ -1,7 +1,8 @@
 // jl_attn_sweep.hip — attention in ONE sweep over the keys (running maximum and sum) on the matrix cores (bfloat16), for heads that
 // come in groups sharing a key head: grouped-query attention, several score maps over the same values, and the single key/value
 // head of latent attention whose values are the first Dv columns of the key rows ([latent | rotary key]).  Sliding window or plain
-// causal; no bias, head mixing or gate (those are jl_attn.hip's).
+// causal, an optional sink in the softmax's denominator and an optional sigmoid gate on the outputs; no bias or head mixing (those
+// are jl_attn.hip's).
 //
 // A workgroup of four wavefronts owns up to 32 rows = (query, head) pairs of one request and one group — HF = min(heads per group,
 // 32) heads of 32 / HF consecutive queries — so a key tile (32 keys through LDS) serves every head of the group at once.  Per tile:
@@ -75,6 +76,8 @@ __global__ __launch_bounds__(AS_THREADS) void attn_sweep_kernel(jl_attn_args a, 
     const int r_i = i0 + rr / HF;
     const bool r_ok = rr < TQ * HF && rr / HF < cnt && h0 + rr % HF < h_end;
     float m_run = -INFINITY, l_run = 0.f;
+    // a sink is a key without a value, counted once: the row's statistics start from it (in the first share of the keys only)
+    if (a.sink && r_ok && blockIdx.z == 0) { m_run = a.sink[h0 + rr % HF]; l_run = 1.f; }
 
     as_f32x16 acc[NT];
 #pragma unroll
@@ -223,8 +226,10 @@ __global__ __launch_bounds__(AS_THREADS) void attn_sweep_kernel(jl_attn_args a, 
             const int col = 32 * (AS_WAVES * t + wave) + l32;
             if (col - l32 >= Dv) continue;
             const int64_t o = ((int64_t)(row0 + ii) * H + hh) * Dv + col;
-            if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[o] = acc[t][r] * inv;
-            else st_f(out + o, acc[t][r] * inv);
+            float v = acc[t][r] * inv;
+            if (a.gate) v *= 1.0f / (1.0f + __expf(-ld_f((const bf16_t *)a.gate + (int64_t)(row0 + ii) * a.gate_ld + (a.gate_heads ? hh : hh * Dv + col))));
+            if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[o] = v;
+            else st_f(out + o, v);
         }
     }
 }
@@ -259,6 +264,7 @@ __global__ __launch_bounds__(256) void attn_sweep_join_kernel(jl_attn_args a, in
         float v = 0.f;
         for (int sp = 0; sp < S; ++sp) v += wS[row * 64 + sp] * base[sp * share + row * (Dv + 2) + col];
         const int64_t o = ((int64_t)(row0 + ii) * H + hh) * Dv + col;
+        if (a.gate) v *= 1.0f / (1.0f + __expf(-ld_f((const bf16_t *)a.gate + (int64_t)(row0 + ii) * a.gate_ld + (a.gate_heads ? hh : hh * Dv + col))));
         if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[o] = v;
         else st_f(out + o, v);
     }

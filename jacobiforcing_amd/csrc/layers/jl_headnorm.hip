@@ -1,5 +1,6 @@
-// jl_headnorm.hip — attention with several score maps per head (differential attention): per-head query / key norm with a
-// position-dependent query temperature and the cache append, and the combination of the maps' outputs.
+// jl_headnorm.hip — per-head query / key stage in front of attention: an optional rotation by position (rotate-half pairs on the first
+// dimensions of every head), the RMS norm of every head's vector (with or without a weight), a position-dependent query temperature,
+// several score maps per head (differential attention), the cache append; and the combination of two maps' outputs.
 #include "jl_common.h"
 
 // One workgroup per token, a wavefront per D-vector (queries first, then keys), then the values.  Vectors are written map-major.
@@ -8,31 +9,39 @@ __global__ __launch_bounds__(256) void head_norm_append_kernel(const T *__restri
                                                                 int M, int D, int GDv, const T *__restrict__ wq, const T *__restrict__ wk, float eps,
                                                                 float t_coef, int t_every, const int32_t *__restrict__ pos, T *__restrict__ q_out,
                                                                 int64_t q_map_stride, T *__restrict__ k_cache, T *__restrict__ v_cache,
-                                                                const int64_t *__restrict__ slot) {
+                                                                const int64_t *__restrict__ slot, int rot_dims, const float *__restrict__ cos_t,
+                                                                const float *__restrict__ sin_t) {
     const int64_t n = blockIdx.x;
     const T *row = proj + n * ld;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t sl = slot[n];
     float temp = 1.0f;
     if (t_coef != 0.f) temp = 1.0f + t_coef * logf((float)((pos[n] + 1) / t_every + 1));
-    const int nq = H * M, nk = G * M;
+    const int nq = H * M, nk = G * M, half = rot_dims / 2;
+    const float *ct = rot_dims ? cos_t + (int64_t)pos[n] * half : nullptr, *sn = rot_dims ? sin_t + (int64_t)pos[n] * half : nullptr;
     for (int vec = wave; vec < nq + nk; vec += 4) {
         const bool is_q = vec < nq;
         const int idx = is_q ? vec : vec - nq;                  // head-major index: head * M + map
         const int head = idx / M, map = idx - head * M;
         const T *src = row + (is_q ? q_col : k_col) + (int64_t)idx * D;
+        // element d after the rotation: (u, v) = (d, d + half) -> (u cos - v sin, v cos + u sin); dimensions from rot_dims on pass
+        auto turned = [&](int d) {
+            const float x = ld_f(src + d);
+            if (d >= rot_dims) return x;
+            return d < half ? x * ct[d] - ld_f(src + d + half) * sn[d] : x * ct[d - half] + ld_f(src + d - half) * sn[d - half];
+        };
         float ss = 0.f;
-        for (int d = lane; d < D; d += 64) { const float v = ld_f(src + d); ss += v * v; }
+        for (int d = lane; d < D; d += 64) { const float v = turned(d); ss += v * v; }
         ss = wave_sum_f32(ss);
         const float r = 1.0f / sqrtf(ss / (float)D + eps);
         if (is_q) {
             // q_map_stride 0: [N, M, H, D]; else [M, N, H, D] with the maps q_map_stride elements apart
             T *dst = q_map_stride ? q_out + map * q_map_stride + n * ((int64_t)H * D) + (int64_t)head * D
                                   : q_out + n * ((int64_t)nq * D) + ((int64_t)map * H + head) * D;
-            for (int d = lane; d < D; d += 64) st_f(dst + d, ld_f(src + d) * r * ld_f(wq + d) * temp);
+            for (int d = lane; d < D; d += 64) st_f(dst + d, turned(d) * r * (wq ? ld_f(wq + d) : 1.0f) * temp);
         } else if (sl >= 0) {
             T *dst = k_cache + sl * ((int64_t)nk * D) + ((int64_t)map * G + head) * D;
-            for (int d = lane; d < D; d += 64) st_f(dst + d, ld_f(src + d) * r * ld_f(wk + d));
+            for (int d = lane; d < D; d += 64) st_f(dst + d, turned(d) * r * (wk ? ld_f(wk + d) : 1.0f));
         }
     }
     if (sl >= 0)
@@ -60,14 +69,27 @@ __global__ __launch_bounds__(256) void head_norm_append_vec_kernel(const T *__re
                                                                     int M, int D, int GDv, const T *__restrict__ wq, const T *__restrict__ wk, float eps,
                                                                     float t_coef, int t_every, const int32_t *__restrict__ pos, T *__restrict__ q_out,
                                                                     int64_t q_map_stride, T *__restrict__ k_cache, T *__restrict__ v_cache,
-                                                                    const int64_t *__restrict__ slot, int LPV) {
+                                                                    const int64_t *__restrict__ slot, int LPV, int rot_dims,
+                                                                    const float *__restrict__ cos_t, const float *__restrict__ sin_t) {
     const int64_t n = blockIdx.x;
     const T *row = proj + n * ld;
     const int sub = threadIdx.x & (LPV - 1), group = threadIdx.x / LPV, groups = 256 / LPV;
     const int64_t sl = slot[n];
     float temp = 1.0f;
     if (t_coef != 0.f) temp = 1.0f + t_coef * logf((float)((pos[n] + 1) / t_every + 1));
-    const int nq = H * M, nk = G * M, d = 4 * sub;
+    const int nq = H * M, nk = G * M, d = 4 * sub, half = rot_dims / 2;
+    // the rotation's pairs (i, i + half) lie four-element groups apart (half % 4 == 0): this lane's partner group and its angles
+    const bool turn = d < rot_dims;
+    const int pd = d < half ? d + half : d - half;
+    float cs[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
+    if (turn) {
+        const int64_t a0 = (int64_t)pos[n] * half + (d < half ? d : d - half);
+        ld4(cos_t + a0, cs);
+        ld4(sin_t + a0, sn);
+        if (d < half)                                           // first of a pair: u cos - v sin; second: v cos + u sin
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sn[i] = -sn[i];
+    }
     for (int v0 = 0; v0 < nq + nk; v0 += groups) {              // every lane takes part in the shuffles of its round
         const int vec = v0 + group;
         const bool live = vec < nq + nk && d < D;
@@ -76,12 +98,18 @@ __global__ __launch_bounds__(256) void head_norm_append_vec_kernel(const T *__re
         const int head = idx / M, map = idx - head * M;
         float x[4] = {0.f, 0.f, 0.f, 0.f};
         if (live) ld4(row + (is_q ? q_col : k_col) + (int64_t)idx * D + d, x);
+        if (live && turn) {
+            float p[4];
+            ld4(row + (is_q ? q_col : k_col) + (int64_t)idx * D + pd, p);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[i] = x[i] * cs[i] + p[i] * sn[i];
+        }
         float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
         for (int off = LPV >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
         if (!live) continue;
         const float r = 1.0f / sqrtf(ss / (float)D + eps) * (is_q ? temp : 1.0f);
-        float g[4];
-        ld4((is_q ? wq : wk) + d, g);
+        float g[4] = {1.f, 1.f, 1.f, 1.f};
+        if (is_q ? wq != nullptr : wk != nullptr) ld4((is_q ? wq : wk) + d, g);
 #pragma unroll
         for (int i = 0; i < 4; ++i) x[i] = x[i] * r * g[i];
         if (is_q) {
@@ -99,23 +127,25 @@ __global__ __launch_bounds__(256) void head_norm_append_vec_kernel(const T *__re
 extern "C" int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t H,
                                    int32_t G, int32_t M, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, float t_coef,
                                    int32_t t_every, const int32_t *pos, void *q_out, int32_t maps_apart, void *k_cache, void *v_cache,
-                                   const int64_t *slot, void *stream) {
+                                   const int64_t *slot, int32_t rot_dims, const float *cos_t, const float *sin_t, void *stream) {
     if (N <= 0) return JL_OK;
-    if (!proj || !wq || !wk || !q_out || !k_cache || !v_cache || !slot) return jl_fail(JL_E_INVALID, "jl_head_norm_append: null pointer");
+    if (!proj || !q_out || !k_cache || !v_cache || !slot) return jl_fail(JL_E_INVALID, "jl_head_norm_append: null pointer");
+    if (rot_dims < 0 || rot_dims % 2 || rot_dims > D || (rot_dims && (!pos || !cos_t || !sin_t)))
+        return jl_fail(JL_E_INVALID, "jl_head_norm_append: a rotation needs an even width up to D, positions and angle tables");
     if (H <= 0 || G <= 0 || M <= 0 || D <= 0 || Dv <= 0 || q_col + (int64_t)H * M * D > ld || k_col + (int64_t)G * M * D > ld || v_col + (int64_t)G * Dv > ld)
         return jl_fail(JL_E_INVALID, "jl_head_norm_append: columns do not fit the row stride");
     if (t_coef != 0.f && (!pos || t_every <= 0)) return jl_fail(JL_E_INVALID, "jl_head_norm_append: a query temperature needs positions and a period >= 1");
-    if (D % 4 == 0 && D <= 256 && ld % 4 == 0 && q_col % 4 == 0 && k_col % 4 == 0) {
+    if (D % 4 == 0 && D <= 256 && ld % 4 == 0 && q_col % 4 == 0 && k_col % 4 == 0 && rot_dims % 8 == 0) {
         int lpv = 1;
         while (4 * lpv < D) lpv <<= 1;
         JL_DISPATCH(dtype, head_norm_append_vec_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(
                                (const T *)proj, ld, q_col, k_col, v_col, H, G, M, D, G * Dv, (const T *)wq, (const T *)wk, eps, t_coef, t_every, pos,
-                               (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot, lpv));
+                               (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot, lpv, rot_dims, cos_t, sin_t));
         return jl_check_launch("head_norm_append_vec_kernel");
     }
     JL_DISPATCH(dtype, head_norm_append_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(
                            (const T *)proj, ld, q_col, k_col, v_col, H, G, M, D, G * Dv, (const T *)wq, (const T *)wk, eps, t_coef, t_every, pos,
-                           (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot));
+                           (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot, rot_dims, cos_t, sin_t));
     return jl_check_launch("head_norm_append_kernel");
 }
 

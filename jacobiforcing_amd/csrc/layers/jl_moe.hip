@@ -1,14 +1,37 @@
-// jl_moe.hip — routed experts: the router's choice, the rows grouped by expert, and the two grouped products around relu^2.
+// jl_moe.hip — routed experts: the router's choice (sigmoid scores with a correction, or a softmax renormalised over the chosen), the
+// rows grouped by expert, and the grouped products: up with relu^2 or plain (a gated unit's activation is its own launch), down with
+// the routing weights.
 #include "jl_common.h"
 #include <stdlib.h>
 
 // ---- router: one thread per token ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ logits, const float *__restrict__ correction, int64_t N,
                                                          int E, int top, float scale, int32_t *__restrict__ ids,
-                                                         float *__restrict__ weights) {
+                                                         float *__restrict__ weights, int kind, float renorm_eps) {
     const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (n >= N) return;
     const float *z = logits + n * E;
+    if (kind == JL_ROUTE_SOFTMAX_RENORM) {
+        // scores = softmax over ALL experts; the largest `top` (ties: lowest index); weights = score / (sum of the chosen + renorm_eps)
+        float zmax = -INFINITY, den = 0.f, chosen = 0.f;
+        for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
+        for (int e = 0; e < E; ++e) den += expf(z[e] - zmax);
+        for (int s = 0; s < top; ++s) {
+            int best = -1;
+            float bz = 0.f;
+            for (int e = 0; e < E; ++e) {
+                bool taken = false;
+                for (int p = 0; p < s; ++p) taken |= ids[n * top + p] == e;
+                if (!taken && (best < 0 || z[e] > bz)) { best = e; bz = z[e]; }
+            }
+            const float sc = expf(bz - zmax) / den;
+            ids[n * top + s] = best;
+            weights[n * top + s] = sc;
+            chosen += sc;
+        }
+        for (int s = 0; s < top; ++s) weights[n * top + s] = weights[n * top + s] / (chosen + renorm_eps) * scale;
+        return;
+    }
     for (int s = 0; s < top; ++s) {
         int best = -1;
         float bc = 0.f, bs = 0.f;
@@ -26,10 +49,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
 }
 
 extern "C" int jl_moe_route(const float *logits, const float *correction, int64_t N, int32_t E, int32_t top, float scale, int32_t *ids,
-                            float *weights, void *stream) {
+                            float *weights, int32_t kind, float renorm_eps, void *stream) {
     if (N <= 0) return JL_OK;
     if (!logits || !ids || !weights || E <= 0 || top <= 0 || top > E) return jl_fail(JL_E_INVALID, "jl_moe_route: null pointer or top > experts");
-    moe_route_kernel<<<dim3((unsigned)((N + 255) / 256)), 256, 0, (hipStream_t)stream>>>(logits, correction, N, E, top, scale, ids, weights);
+    if (kind != JL_ROUTE_SIGMOID && kind != JL_ROUTE_SOFTMAX_RENORM) return jl_fail(JL_E_INVALID, "jl_moe_route: unknown kind %d", kind);
+    moe_route_kernel<<<dim3((unsigned)((N + 255) / 256)), 256, 0, (hipStream_t)stream>>>(logits, correction, N, E, top, scale, ids, weights, kind,
+                                                                                         renorm_eps);
     return jl_check_launch("moe_route_kernel");
 }
 
@@ -98,7 +123,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
     const int nr = offsets[e + 1] - r0 < MOE_TM ? offsets[e + 1] - r0 : MOE_TM;
     const int n0 = blockIdx.y * MOE_TN;
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
-    if (tid < MOE_TM) rin[tid] = tid < nr ? (mode == 0 ? perm[r0 + tid] / top : r0 + tid) : -1;
+    if (tid < MOE_TM) rin[tid] = tid < nr ? (mode != 1 ? perm[r0 + tid] / top : r0 + tid) : -1;
     const T *We = Wt + (int64_t)e * n_out * K;
     float acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += MOE_TK) {
@@ -134,7 +159,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
         for (int c = 0; c < 4; ++c) {
             const int n = n0 + tx + 16 * c;
             if (n >= n_out) continue;
-            if (mode == 0) {
+            if (mode == JL_MOE_UP_PLAIN) {
+                st_f((T *)out + (int64_t)r * n_out + n, acc[a][c]);
+            } else if (mode == 0) {
                 const float v = fmaxf(acc[a][c], 0.f);
                 st_f((T *)out + (int64_t)r * n_out + n, v * v);
             } else {
@@ -167,7 +194,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
     const int nr = offsets[e + 1] - r0 < MOE_TM ? offsets[e + 1] - r0 : MOE_TM;
     const int n0 = blockIdx.y * MM_TN;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    if (tid < MOE_TM) rin[tid] = tid < nr ? (mode == 0 ? perm[r0 + tid] / top : r0 + tid) : -1;
+    if (tid < MOE_TM) rin[tid] = tid < nr ? (mode != 1 ? perm[r0 + tid] / top : r0 + tid) : -1;
     __syncthreads();
     const bf16_t *We = Wt + (int64_t)e * n_out * K;
     // loaders: 8 bf16 (16 bytes) per thread and row segment; A 64 x 32 = 256 segments, B 128 x 32 = 512 segments
@@ -222,7 +249,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
             if (m >= nr) continue;
             const float c = half ? acc1[i] : acc0[i];
             const int r = r0 + m;
-            if (mode == 0) {
+            if (mode == JL_MOE_UP_PLAIN) {
+                st_f((bf16_t *)out + (int64_t)r * n_out + n, c);
+            } else if (mode == 0) {
                 const float v = fmaxf(c, 0.f);
                 st_f((bf16_t *)out + (int64_t)r * n_out + n, v * v);
             } else {
@@ -238,7 +267,7 @@ extern "C" int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mod
     if (max_tiles <= 0) return JL_OK;
     if (!X || !Wt || !perm || !offsets || !tile_expert || !tile_row0 || !out || (mode == 1 && !weights))
         return jl_fail(JL_E_INVALID, "jl_moe_gemm: null pointer");
-    if (K <= 0 || n_out <= 0 || top <= 0 || (mode != 0 && mode != 1)) return jl_fail(JL_E_INVALID, "jl_moe_gemm: bad sizes or mode");
+    if (K <= 0 || n_out <= 0 || top <= 0 || (mode != 0 && mode != 1 && mode != JL_MOE_UP_PLAIN)) return jl_fail(JL_E_INVALID, "jl_moe_gemm: bad sizes or mode");
     static const bool no_mfma = getenv("JL_MOE_NO_MFMA") != nullptr;      // A/B switch for measurements
     if (!no_mfma && dtype == JL_BF16 && K % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0) {
         const dim3 mgrid((unsigned)max_tiles, (unsigned)((n_out + MM_TN - 1) / MM_TN));

@@ -57,6 +57,89 @@ extern "C" int jl_add_rmsnorm(float *x, const void *y, int y_dtype, int32_t y_co
     return jl_check_launch("add_rmsnorm_kernel");
 }
 
+// ---- several scaled addends + up to two norms of the same row (a layer whose sublayers all read one stream) ---------------------------------
+// pass 1: x += sum_a scale_a * (sum over the addend's middle axis), written back, with the sum of squares; pass 2: both outputs
+template <typename T>
+__global__ __launch_bounds__(256) void scaled_add_norms_kernel(float *__restrict__ x, jl_addend a0, jl_addend a1, jl_addend a2, const float *__restrict__ w1,
+                                                                const float *__restrict__ w2, float w_offset, float eps, T *__restrict__ out1,
+                                                                T *__restrict__ out2, int W) {
+    __shared__ float red[16];
+    const int64_t n = blockIdx.x;
+    float *xr = x + n * W;
+    const jl_addend ad[3] = {a0, a1, a2};
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            if (!ad[k].y) continue;
+            float u = 0.f;
+            for (int s = 0; s < ad[k].count; ++s) u += ld_any(ad[k].y, ad[k].dtype, (n * ad[k].count + s) * (int64_t)W + c);
+            t += ad[k].scale ? u * ad[k].scale[c] : u;
+        }
+        const float v = xr[c] + t;
+        if (a0.y || a1.y || a2.y) xr[c] = v;
+        ss += v * v;
+    }
+    if (!out1 && !out2) return;
+    ss = block_sum_f32(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float v = xr[c] * r;
+        if (out1) st_f(out1 + n * W + c, w1 ? v * (w_offset + w1[c]) : v);
+        if (out2) st_f(out2 + n * W + c, w2 ? v * (w_offset + w2[c]) : v);
+    }
+}
+
+extern "C" int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n_addends, const float *w1, const float *w2, float w_offset, float eps,
+                                   void *out1, void *out2, int dtype, int64_t N, int32_t W, void *stream) {
+    if (N <= 0) return JL_OK;
+    if (!x || W <= 0 || n_addends < 0 || n_addends > 3 || (n_addends && !addends)) return jl_fail(JL_E_INVALID, "jl_scaled_add_norms: null pointer, bad width or more than 3 addends");
+    jl_addend ad[3] = {{nullptr, 0, 0, nullptr}, {nullptr, 0, 0, nullptr}, {nullptr, 0, 0, nullptr}};
+    for (int k = 0; k < n_addends; ++k) {
+        ad[k] = addends[k];
+        if (ad[k].y && ad[k].count <= 0) return jl_fail(JL_E_INVALID, "jl_scaled_add_norms: addend %d has no rows", k);
+    }
+    JL_DISPATCH(dtype, scaled_add_norms_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x, ad[0], ad[1], ad[2], w1, w2, w_offset, eps, (T *)out1,
+                                                                                                      (T *)out2, W));
+    return jl_check_launch("scaled_add_norms_kernel");
+}
+
+// ---- gated activation of a feed-forward: out[n, c] = act(z[n, g_col + c]) * lin(z[n, u_col + c]) (* sigmoid(row_gate[n])) -----------------
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename T>
+__global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ z, int64_t ld, int g_col, int u_col, int F, int kind, float limit, float alpha,
+                                                         float shift, const T *__restrict__ row_gate, int64_t rg_ld, T *__restrict__ out, int64_t total) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    const int64_t n = e / F;
+    const int c = (int)(e - n * F);
+    float g = ld_f(z + n * ld + g_col + c), u = ld_f(z + n * ld + u_col + c), v;
+    if (kind == JL_ACT_GELU_TANH) {
+        v = gelu_tanh_f(g) * u;
+    } else {                                                        // clamped swish: the gate capped from above, the linear branch from both sides
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        v = g / (1.0f + expf(-alpha * g)) * (u + shift);
+    }
+    if (row_gate) v *= 1.0f / (1.0f + expf(-ld_f(row_gate + n * rg_ld)));
+    st_f(out + e, v);
+}
+
+extern "C" int jl_gated_act(const void *z, int dtype, int64_t N, int64_t ld, int32_t g_col, int32_t u_col, int32_t F, int32_t kind, float limit, float alpha,
+                            float shift, const void *row_gate, int64_t rg_ld, void *out, void *stream) {
+    if (N <= 0) return JL_OK;
+    if (!z || !out || F <= 0 || g_col < 0 || u_col < 0 || g_col + (int64_t)F > ld || u_col + (int64_t)F > ld)
+        return jl_fail(JL_E_INVALID, "jl_gated_act: null pointer, or the columns do not fit the row stride");
+    if (kind != JL_ACT_GELU_TANH && kind != JL_ACT_CLAMPED_SWISH) return jl_fail(JL_E_INVALID, "jl_gated_act: unknown kind %d", kind);
+    const int64_t total = N * F;
+    JL_DISPATCH(dtype, gated_act_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0, (hipStream_t)stream>>>(
+                           (const T *)z, ld, g_col, u_col, F, kind, limit, alpha, shift, (const T *)row_gate, rg_ld, (T *)out, total));
+    return jl_check_launch("gated_act_kernel");
+}
+
 // ---- sublayer-output norm + residual update: one workgroup per row ------------------------------------------------------------
 template <typename TY, typename TO>
 __global__ __launch_bounds__(256) void norm_add_kernel(float *__restrict__ x, const TY *__restrict__ y, const float *__restrict__ g, float eps,

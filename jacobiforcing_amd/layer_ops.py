@@ -177,6 +177,14 @@ def qk_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: in
     return q
 
 
+def _check_gate_sink(gate, sink, gate_per_head: bool, n: int, H: int, Dv: int, dt, what: str) -> None:
+    if gate is not None:
+        _need(gate.shape == (n, H if gate_per_head else H * Dv) and gate.stride(1) == 1 and gate.dtype == dt,
+              f"{what}: gate [N, H*Dv], or [N, H] with one gate per head")
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == H, f"{what}: sink float [H]")
+
+
 def attn_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int, k_ld: int = 0, v_ld: int = 0) -> int:
     tq = int(N.layers().jl_attn_tile_rows(_code(dtype), H, G, D, Dv, k_ld, v_ld))
     if tq <= 0:
@@ -186,8 +194,10 @@ def attn_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int, k_ld: in
 
 def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, batch: RaggedBatch,
                 H: int, G: int, D: int, Dv: int, scale: float, window: int, keep_first: int, rel: Optional[torch.Tensor],
-                lut: Optional[torch.Tensor], talk: Optional[torch.Tensor], value_heads: int = 0, float_out: bool = False) -> torch.Tensor:
-    """q [N, H*D]; gate a [N, H*Dv] view (column range of the projection output, row stride free) or None.  Returns [N, H*Dv].
+                lut: Optional[torch.Tensor], talk: Optional[torch.Tensor], value_heads: int = 0, float_out: bool = False,
+                sink: Optional[torch.Tensor] = None, gate_per_head: bool = False) -> torch.Tensor:
+    """q [N, H*D]; gate a [N, H*Dv] view (column range of the projection output, row stride free; [N, H] with ``gate_per_head``) or
+    None.  ``sink`` float [H]: one more term exp(sink_h) in every softmax denominator of head h.  Returns [N, H*Dv].
     The pools may be column ranges of wider rows (``v_cache`` may be a view into ``k_cache``).  ``value_heads`` (0: G) < G: key head
     c reads value head c % value_heads — several score maps over the same values.  ``float_out``: float outputs from bfloat16
     inputs (for what is subtracted or normalised next)."""
@@ -202,8 +212,7 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
     k_ld, v_ld = k_cache.stride(0), v_cache.stride(0)
     pool_tokens = k_cache.shape[0]
     _need(pool_tokens % batch.page_size == 0 and batch.max_page < pool_tokens // batch.page_size, "attn_window: a page lies outside the pool")
-    if gate is not None:
-        _need(gate.shape == (n, H * Dv) and gate.stride(1) == 1 and gate.dtype == dt, "attn_window: gate [N, H*Dv]")
+    _check_gate_sink(gate, sink, gate_per_head, n, H, Dv, dt, "attn_window")
     for t, shape in ((rel, None), (talk, (H, H))):
         if t is not None:
             _need(t.dtype == torch.float32 and t.is_contiguous() and (shape is None or tuple(t.shape) == shape), "attn_window: float tables")
@@ -228,7 +237,8 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
                    keep_first=int(keep_first), TQ=tq, dtype=_code(dt), scale=float(scale), splits=splits, n_rows=n,
                    scratch=scratch.data_ptr() if scratch is not None else None,
                    q_pack=q_pack.data_ptr() if q_pack is not None else None, k_ld=k_ld, v_ld=v_ld, Gv=Gv,
-                   out_dtype=N.JL_OUT_F32 if float_out and dt != torch.float32 else N.JL_OUT_SAME)
+                   out_dtype=N.JL_OUT_F32 if float_out and dt != torch.float32 else N.JL_OUT_SAME,
+                   sink=sink.data_ptr() if sink is not None else None, gate_heads=int(gate_per_head))
     N.check_layers(N.layers().jl_attn_window(C.byref(a), _stream(q.device)), "jl_attn_window")
     return out
 
@@ -243,8 +253,9 @@ def attn_sweep_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int, k_
 
 
 def attn_sweep(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, batch: RaggedBatch, H: int, G: int, D: int, Dv: int, scale: float,
-               window: int, value_heads: int = 0, float_out: bool = False) -> torch.Tensor:
-    """Attention without bias, head mixing or gate in one sweep on the matrix cores: q [N, H*D] bfloat16, pools as for
+               window: int, value_heads: int = 0, float_out: bool = False, sink: Optional[torch.Tensor] = None,
+               gate: Optional[torch.Tensor] = None, gate_per_head: bool = False) -> torch.Tensor:
+    """Attention without bias or head mixing (``sink`` / ``gate`` as for ``attn_window``) in one sweep on the matrix cores: q [N, H*D] bfloat16, pools as for
     ``attn_window`` (column ranges of wider rows allowed); ``v_cache`` may be the first Dv columns of ``k_cache`` itself (one key
     head whose rows hold the values: the latent pool).  Returns [N, H*Dv].  Sizes as ``attn_sweep_tile_rows`` accepts them."""
     _dev(q)
@@ -255,6 +266,7 @@ def attn_sweep(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ba
           v_cache.shape[1] == Gv * Dv and k_cache.stride(1) == 1 and v_cache.stride(1) == 1 and k_cache.shape[0] == v_cache.shape[0],
           "attn_sweep: pool dtype / widths")
     _need(k_cache.shape[0] % batch.page_size == 0 and batch.max_page < k_cache.shape[0] // batch.page_size, "attn_sweep: a page lies outside the pool")
+    _check_gate_sink(gate, sink, gate_per_head, n, H, Dv, q.dtype, "attn_sweep")
     tq = attn_sweep_tile_rows(q.dtype, H, G, D, Dv, k_cache, v_cache, Gv)
     _need(tq > 0, f"attn_sweep: heads={H} kv_heads={G} dim={D} vdim={Dv} are not sizes of this kernel")
     tiles = batch.tiles(tq)
@@ -271,7 +283,8 @@ def attn_sweep(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ba
                    tiles=tiles.data_ptr(), bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0], page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv,
                    window=int(window), TQ=tq, dtype=_code(q.dtype), scale=float(scale), n_rows=n, k_ld=k_cache.stride(0), v_ld=v_cache.stride(0), Gv=Gv,
                    splits=splits, scratch=scratch.data_ptr() if scratch is not None else None,
-                   out_dtype=N.JL_OUT_F32 if float_out else N.JL_OUT_SAME)
+                   out_dtype=N.JL_OUT_F32 if float_out else N.JL_OUT_SAME, sink=sink.data_ptr() if sink is not None else None,
+                   gate=gate.data_ptr() if gate is not None else None, gate_ld=gate.stride(0) if gate is not None else 0, gate_heads=int(gate_per_head))
     N.check_layers(N.layers().jl_attn_sweep(C.byref(a), _stream(q.device)), "jl_attn_sweep")
     return out
 
@@ -312,23 +325,32 @@ def retention(proj: torch.Tensor, cols: Tuple[int, int, int, int], batch: Ragged
 
 
 def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, scale: float,
-                w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
-    """Routed experts down(relu(up h)^2): h [N, W], router_logits float [N, E], w_up [E, ff, W], w_down [E, W, ff].  Returns the
-    weighted expert outputs per choice, float [N, top, W] (their sum over the middle axis is the layer's output)."""
+                w_up: torch.Tensor, w_down: torch.Tensor, route: str = "sigmoid", renorm_eps: float = 0.0,
+                gated: Optional[Tuple[int, float, float, float]] = None) -> torch.Tensor:
+    """Routed experts: h [N, W], router_logits float [N, E], w_down [E, W, ff].  Returns the weighted expert outputs per choice,
+    float [N, top, W] (their sum over the middle axis is the layer's output).
+
+    ``route`` "sigmoid": sigmoid scores, choice by score + correction, weights = score * scale; "softmax_renorm": softmax over all
+    experts, the largest chosen, weights = score / (sum of the chosen + renorm_eps) * scale.
+    ``gated`` None: experts down(relu(up h)^2) with w_up [E, ff, W].  ``gated`` = (kind, limit, alpha, shift) of ``gated_act``: w_up
+    [E, 2*ff, W] stacks every expert's gate rows on its linear rows, and the activation is a launch between the two products."""
     _dev(h)
     n, W = h.shape
-    E, ff = w_up.shape[0], w_up.shape[1]
+    E, ff = w_down.shape[0], w_down.shape[2]
+    up_rows = 2 * ff if gated is not None else ff
     dev, dt = h.device, h.dtype
     _need(h.is_contiguous() and router_logits.dtype == torch.float32 and router_logits.is_contiguous() and tuple(router_logits.shape) == (n, E),
           "moe_experts: h [N, W], logits float [N, E]")
-    _need(tuple(w_up.shape) == (E, ff, W) and tuple(w_down.shape) == (E, W, ff) and w_up.dtype == dt and w_down.dtype == dt and
-          w_up.is_contiguous() and w_down.is_contiguous(), "moe_experts: expert weights [E, ff, W] / [E, W, ff] in the activation dtype")
+    _need(tuple(w_up.shape) == (E, up_rows, W) and tuple(w_down.shape) == (E, W, ff) and w_up.dtype == dt and w_down.dtype == dt and
+          w_up.is_contiguous() and w_down.is_contiguous(), "moe_experts: expert weights [E, ff (2*ff when gated), W] / [E, W, ff] in the activation dtype")
+    _need(route in ("sigmoid", "softmax_renorm") and 1 <= top <= E, "moe_experts: route is 'sigmoid' or 'softmax_renorm', 1 <= top <= experts")
     if correction is not None:
         _need(correction.dtype == torch.float32 and correction.numel() == E, "moe_experts: correction float [E]")
     L, st = N.layers(), _stream(dev)
     ids = torch.empty((n, top), dtype=torch.int32, device=dev)
     wts = torch.empty((n, top), dtype=torch.float32, device=dev)
-    N.check_layers(L.jl_moe_route(_ptr(router_logits), _ptr(correction), n, E, top, float(scale), _ptr(ids), _ptr(wts), st), "jl_moe_route")
+    N.check_layers(L.jl_moe_route(_ptr(router_logits), _ptr(correction), n, E, top, float(scale), _ptr(ids), _ptr(wts),
+                                  N.JL_ROUTE_SIGMOID if route == "sigmoid" else N.JL_ROUTE_SOFTMAX_RENORM, float(renorm_eps), st), "jl_moe_route")
     tm = int(L.jl_moe_tile_rows())
     rows = n * top
     max_tiles = rows // tm + E
@@ -337,13 +359,61 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
     tile_e = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
     tile_r = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
     N.check_layers(L.jl_moe_group(_ptr(ids), n, top, E, tm, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles, st), "jl_moe_group")
-    act = torch.empty((rows, ff), dtype=dt, device=dev)
-    N.check_layers(L.jl_moe_gemm(_ptr(h), _ptr(w_up), _code(dt), 0, W, ff, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
-                                 None, _ptr(act), st), "jl_moe_gemm(up)")
+    act = torch.empty((rows, up_rows), dtype=dt, device=dev)
+    N.check_layers(L.jl_moe_gemm(_ptr(h), _ptr(w_up), _code(dt), N.JL_MOE_UP_PLAIN if gated is not None else N.JL_MOE_UP_RELU2, W, up_rows, top, _ptr(perm),
+                                 _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles, None, _ptr(act), st), "jl_moe_gemm(up)")
+    if gated is not None:
+        act = gated_act(act, 0, ff, ff, *gated)
     y = torch.empty((n, top, W), dtype=torch.float32, device=dev)
-    N.check_layers(L.jl_moe_gemm(_ptr(act), _ptr(w_down), _code(dt), 1, ff, W, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
+    N.check_layers(L.jl_moe_gemm(_ptr(act), _ptr(w_down), _code(dt), N.JL_MOE_DOWN, ff, W, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
                                  _ptr(wts), _ptr(y), st), "jl_moe_gemm(down)")
     return y
+
+
+ACT_GELU_TANH, ACT_CLAMPED_SWISH = N.JL_ACT_GELU_TANH, N.JL_ACT_CLAMPED_SWISH
+
+
+def gated_act(z: torch.Tensor, g_col: int, u_col: int, F_: int, kind: int, limit: float = 0.0, alpha: float = 1.0, shift: float = 0.0,
+              row_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gated activation of a feed-forward whose gate and linear branch are F_ columns each of one product z [N, ld], at g_col /
+    u_col.  ACT_GELU_TANH: gelu_tanh(g) * u.  ACT_CLAMPED_SWISH: g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(alpha g') (u' +
+    shift).  ``row_gate`` [N] or [N, 1] view (row stride free): the row is further multiplied by sigmoid(row_gate).  Returns [N, F_]."""
+    _dev(z)
+    _need(z.dim() == 2 and z.stride(1) == 1 and g_col + F_ <= z.shape[1] and u_col + F_ <= z.shape[1], "gated_act: z [N, ld] with both column ranges inside")
+    n = z.shape[0]
+    rg_ld = 0
+    if row_gate is not None:
+        _need(row_gate.dtype == z.dtype and row_gate.numel() == n and row_gate.shape[0] == n, "gated_act: one row gate per row, of z's dtype")
+        rg_ld = row_gate.stride(0)
+    out = torch.empty((n, F_), dtype=z.dtype, device=z.device)
+    N.check_layers(N.layers().jl_gated_act(_ptr(z), _code(z.dtype), n, z.stride(0), g_col, u_col, F_, int(kind), float(limit), float(alpha), float(shift),
+                                          _ptr(row_gate), rg_ld, _ptr(out), _stream(z.device)), "jl_gated_act")
+    return out
+
+
+def scaled_add_norms(x: torch.Tensor, addends: Sequence[Tuple[torch.Tensor, Optional[torch.Tensor]]], w1: Optional[torch.Tensor],
+                     w2: Optional[torch.Tensor], w_offset: float, eps: float, out_dtype: Optional[torch.dtype], two: bool = False):
+    """x (float [N, W], in place) += sum over ``addends`` (y, scale) of scale * y, y [N, W] or [N, S, W] (summed over S) float or
+    bfloat16, scale float [W] or None; then, with ``out_dtype``, the RMS norm of the updated x with float weights stored around
+    ``w_offset``: x / rms(x) * (w_offset + w1) — and the same with w2 when ``two`` (both sublayers of a layer read one stream).
+    Returns None, the norm, or the pair of norms."""
+    _dev(x)
+    n, W = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and len(addends) <= 3, "scaled_add_norms: x contiguous float32 [N, W], at most 3 addends")
+    arr = (N.Addend * max(1, len(addends)))()
+    for k, (y, sc) in enumerate(addends):
+        _need(y.is_contiguous() and y.shape[0] == n and y.shape[-1] == W and y.dim() in (2, 3), "scaled_add_norms: an addend is [N, W] or [N, S, W]")
+        if sc is not None:
+            _need(sc.dtype == torch.float32 and sc.numel() == W and sc.is_contiguous(), "scaled_add_norms: a scale is float [W]")
+        arr[k] = N.Addend(y=y.data_ptr(), dtype=_code(y.dtype), count=1 if y.dim() == 2 else y.shape[1], scale=sc.data_ptr() if sc is not None else None)
+    for w in (w1, w2):
+        if w is not None:
+            _need(w.dtype == torch.float32 and w.numel() == W and w.is_contiguous(), "scaled_add_norms: norm weights are float [W]")
+    out1 = torch.empty((n, W), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    out2 = torch.empty((n, W), dtype=out_dtype, device=x.device) if out_dtype is not None and two else None
+    N.check_layers(N.layers().jl_scaled_add_norms(_ptr(x), arr, len(addends), _ptr(w1), _ptr(w2), float(w_offset), float(eps), _ptr(out1), _ptr(out2),
+                                                 _code(out_dtype or torch.float32), n, W, _stream(x.device)), "jl_scaled_add_norms")
+    return (out1, out2) if two else out1
 
 
 def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, out_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
@@ -388,23 +458,30 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, batch: RaggedBatch, tail: Opti
     return out
 
 
-def head_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: int, M: int, D: int, Dv: int, wq: torch.Tensor, wk: torch.Tensor,
-                     eps: float, t_coef: float, t_every: int, batch: RaggedBatch, k_cache: torch.Tensor, v_cache: torch.Tensor,
-                     maps_apart: bool = False) -> torch.Tensor:
-    """Per-head (and per score map) RMS norm of q and k over D, query temperature by position, keys / values appended to the
+def head_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: int, M: int, D: int, Dv: int, wq: Optional[torch.Tensor],
+                     wk: Optional[torch.Tensor], eps: float, t_coef: float, t_every: int, batch: RaggedBatch, k_cache: torch.Tensor,
+                     v_cache: torch.Tensor, maps_apart: bool = False, rot_dims: int = 0, cos: Optional[torch.Tensor] = None,
+                     sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per-head (and per score map) stage in front of attention: with ``rot_dims`` the rotation of q and k by position (rotate-half
+    pairs on the first rot_dims dimensions of every head, angles from cos / sin [positions, rot_dims / 2] float), then the RMS norm
+    of q and k over D (times wq / wk [D]; None: no weight), the query temperature by position, keys / values appended to the
     pools.  Returns q [N, M*H*D] map-major ([M, N, H*D] with ``maps_apart``: a contiguous query matrix per map); the key pool rows
     are [M, G, D] map-major."""
     _dev(proj)
     n, ld = proj.shape
     dt = proj.dtype
     _need(proj.is_contiguous() and n == batch.N, "head_norm_append: proj [N, ld] of the batch")
-    _need(wq.numel() == D and wk.numel() == D and wq.dtype == dt and wk.dtype == dt, "head_norm_append: norm weights over one head")
+    for w in (wq, wk):
+        _need(w is None or (w.numel() == D and w.dtype == dt), "head_norm_append: norm weights over one head")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= D, "head_norm_append: the rotation takes an even number of dimensions up to D")
+    _angle_tables(rot_dims, cos, sin, batch, "head_norm_append")
     _need(k_cache.dtype == dt and v_cache.dtype == dt and k_cache.is_contiguous() and v_cache.is_contiguous() and
           k_cache.shape[-1] == M * G * D and v_cache.shape[-1] == G * Dv and k_cache.shape[0] == v_cache.shape[0], "head_norm_append: pools [tokens, M*G*D] / [tokens, G*Dv]")
     q = torch.empty((M, n, H * D) if maps_apart else (n, M * H * D), dtype=dt, device=proj.device)
     N.check_layers(N.layers().jl_head_norm_append(_ptr(proj), _code(dt), n, ld, cols[0], cols[1], cols[2], H, G, M, D, Dv, _ptr(wq), _ptr(wk), float(eps),
                                                  float(t_coef), int(t_every), _ptr(batch.pos), _ptr(q), int(maps_apart), _ptr(k_cache), _ptr(v_cache),
-                                                 _ptr(batch.kv_slot), _stream(proj.device)), "jl_head_norm_append")
+                                                 _ptr(batch.kv_slot), int(rot_dims), _ptr(cos) if rot_dims else None, _ptr(sin) if rot_dims else None,
+                                                 _stream(proj.device)), "jl_head_norm_append")
     return q
 
 

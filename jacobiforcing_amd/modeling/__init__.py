@@ -14,6 +14,7 @@ MODEL_REGISTRY = {
     "Qwen2ForCausalLM": ("jacobiforcing_amd.modeling.qwen2", "Qwen2Config", "padded"),
     "Lokizen": ("jacobiforcing_amd.modeling.lokizen", "LokizenConfig", "ragged"),
     "Vumalix": ("jacobiforcing_amd.modeling.vumalix", "VumalixConfig", "ragged"),
+    "Bamanex": ("jacobiforcing_amd.modeling.bamanex", "BamanexConfig", "ragged"),
 }
 
 
