@@ -35,20 +35,14 @@ def gelu_tanh(z):
 def stretched_frequencies(dims: int, base: float, scaling) -> list:
     """f_i = base^(-2i/dims), i < dims/2; with ``scaling`` {factor, low, high, original}: a frequency whose wavelength is shorter
     than original/high stays, one longer than original/low is divided by factor, and between the two the result slides from the
-    divided to the kept frequency with s = (original/wavelength - low) / (high - low)."""
-    out = []
-    for i in range(dims // 2):
-        f = base ** (-2.0 * i / dims)
-        if scaling:
-            factor, low, high, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
-            wl = 2.0 * math.pi / f
-            if wl > orig / low:
-                f = f / factor
-            elif wl >= orig / high:
-                s = (orig / wl - low) / (high - low)
-                f = (1.0 - s) * f / factor + s * f
-        out.append(f)
-    return out
+    divided to the kept frequency with s = (original/wavelength - low) / (high - low).  Written over the whole vector at once."""
+    f = torch.tensor(float(base), dtype=torch.float64) ** (-torch.arange(0, dims, 2, dtype=torch.float64) / dims)
+    if scaling:
+        factor, low, high, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+        turns = orig * f / (2.0 * math.pi)                               # how often the pair goes round within `original` positions
+        s = ((turns - low) / (high - low)).clamp(0.0, 1.0)               # 0: long wavelengths, 1: short ones
+        f = (1.0 - s) * f / factor + s * f
+    return f.tolist()
 
 
 def rotate_pairs(vec, position: int, freqs):
