@@ -218,6 +218,13 @@ JL_API int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mode, i
                        const int32_t *perm, const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0,
                        int32_t max_tiles, const float *weights, void *out, void *stream);
 
+/* The up product of gated experts with the unit applied in its epilogue: W [E, 2*ff, K] stacks every expert's gate rows on its
+ * linear rows; out[r, c] = unit(X[in(r)] . W[e(r), c], X[in(r)] . W[e(r), ff + c]) with in(r) = perm[r] / top, stored in `dtype`
+ * ([N*top, ff], sorted order); kind / limit / alpha / shift as for jl_gated_act. */
+JL_API int jl_moe_gemm_gated(const void *X, const void *Wt, int dtype, int32_t K, int32_t ff, int32_t top, const int32_t *perm,
+                             const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0, int32_t max_tiles, int32_t kind,
+                             float limit, float alpha, float shift, void *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

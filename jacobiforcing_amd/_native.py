@@ -284,10 +284,11 @@ _LAYER_SIGNATURES = {
     "jl_moe_group": (C.c_int, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp]),
     "jl_moe_tile_rows": (C.c_int, []),
     "jl_moe_gemm": (C.c_int, [_vp, _vp, C.c_int, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
+    "jl_moe_gemm_gated": (C.c_int, [_vp, _vp, C.c_int, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _f32, _f32, _f32, _vp, _vp]),
 }
 LAYER_SYMBOLS = tuple(_LAYER_SIGNATURES)
 # which library a symbol lives in (jacobiforcing_amd/_build.py: LAYER_GROUPS); both carry their own jl_version / jl_last_error
-_SEQ_SYMBOLS = ("jl_retention", "jl_retention_join", "jl_moe_route", "jl_moe_group", "jl_moe_tile_rows", "jl_moe_gemm")
+_SEQ_SYMBOLS = ("jl_retention", "jl_retention_join", "jl_moe_route", "jl_moe_group", "jl_moe_tile_rows", "jl_moe_gemm", "jl_moe_gemm_gated")
 
 
 class _LayerLibs:

@@ -50,6 +50,18 @@ __device__ __forceinline__ float block_sum_f32(float v, float *red) {
     return s;
 }
 
+// gated units of a feed-forward (jl_gated_act, and the grouped product that applies them in its epilogue)
+// 0.5 z (1 + tanh(u)) = z sigmoid(2u), u = sqrt(2/pi) (z + 0.044715 z^3)
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    return z / (1.0f + expf(-1.5957691216057308f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float gated_unit_f(float g, float u, int kind, float limit, float alpha, float shift) {
+    if (kind == JL_ACT_GELU_TANH) return gelu_tanh_f(g) * u;
+    g = fminf(g, limit);                                            // clamped swish: the gate capped from above, the linear branch from both sides
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-alpha * g)) * (u + shift);
+}
+
 #define JL_DISPATCH(dtype, ...)                                   \
     do {                                                          \
         if ((dtype) == JL_BF16) { typedef bf16_t T; __VA_ARGS__; } \

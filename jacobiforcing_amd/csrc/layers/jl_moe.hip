@@ -109,13 +109,16 @@ extern "C" int jl_moe_group(const int32_t *ids, int64_t N, int32_t top, int32_t 
 }
 
 // ---- grouped product, any dtype and size: a 64 x 64 tile of one expert's rows per workgroup, float FMAs ------------------------------------
-template <typename T>
+struct MoeAct { int kind; float limit, alpha, shift; };       // the gated unit of JL_MOE_UP_GATED (jl_gated_act's kinds)
+
+// GATED: W holds 2 * n_out rows per expert, gate rows on linear rows; a tile forms both products of its columns and stores the unit
+template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, const T *__restrict__ Wt, int mode, int K, int n_out, int top,
                                                         const int32_t *__restrict__ perm, const int32_t *__restrict__ offsets,
                                                         const int32_t *__restrict__ tile_expert, const int32_t *__restrict__ tile_row0,
-                                                        const float *__restrict__ weights, void *__restrict__ out) {
+                                                        const float *__restrict__ weights, void *__restrict__ out, MoeAct act) {
     __shared__ float Xs[MOE_TM][MOE_TK + 1];
-    __shared__ float Ws[MOE_TN][MOE_TK + 1];
+    __shared__ float Ws[(GATED ? 2 : 1) * MOE_TN][MOE_TK + 1];
     __shared__ int rin[MOE_TM];
     const int e = tile_expert[blockIdx.x];
     if (e < 0) return;
@@ -124,8 +127,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
     const int n0 = blockIdx.y * MOE_TN;
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
     if (tid < MOE_TM) rin[tid] = tid < nr ? (mode != 1 ? perm[r0 + tid] / top : r0 + tid) : -1;
-    const T *We = Wt + (int64_t)e * n_out * K;
+    const T *We = Wt + (int64_t)e * (GATED ? 2 : 1) * n_out * K;
     float acc[4][4] = {};
+    float acu[GATED ? 4 : 1][4] = {};
     for (int k0 = 0; k0 < K; k0 += MOE_TK) {
         __syncthreads();
         for (int i = tid; i < MOE_TM * MOE_TK; i += 256) {
@@ -135,6 +139,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
         for (int i = tid; i < MOE_TN * MOE_TK; i += 256) {
             const int n = i / MOE_TK, kk = i - n * MOE_TK;
             Ws[n][kk] = (n0 + n < n_out && k0 + kk < K) ? ld_f(We + (int64_t)(n0 + n) * K + k0 + kk) : 0.f;
+            if (GATED) Ws[MOE_TN + n][kk] = (n0 + n < n_out && k0 + kk < K) ? ld_f(We + (int64_t)(n_out + n0 + n) * K + k0 + kk) : 0.f;
         }
         __syncthreads();
 #pragma unroll 8
@@ -147,6 +152,11 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
                 const float w = Ws[tx + 16 * c][kk];
 #pragma unroll
                 for (int a = 0; a < 4; ++a) acc[a][c] += av[a] * w;
+                if (GATED) {
+                    const float wu = Ws[MOE_TN + tx + 16 * c][kk];
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) acu[GATED ? a : 0][c] += av[a] * wu;
+                }
             }
         }
     }
@@ -159,7 +169,9 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
         for (int c = 0; c < 4; ++c) {
             const int n = n0 + tx + 16 * c;
             if (n >= n_out) continue;
-            if (mode == JL_MOE_UP_PLAIN) {
+            if (GATED) {
+                st_f((T *)out + (int64_t)r * n_out + n, gated_unit_f(acc[a][c], acu[GATED ? a : 0][c], act.kind, act.limit, act.alpha, act.shift));
+            } else if (mode == JL_MOE_UP_PLAIN) {
                 st_f((T *)out + (int64_t)r * n_out + n, acc[a][c]);
             } else if (mode == 0) {
                 const float v = fmaxf(acc[a][c], 0.f);
@@ -181,12 +193,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 constexpr int MM_TN = 128, MM_TK = 32, MM_LD = 36;     // LDS row stride in bf16 (72 bytes: rows 16 apart share a bank, no worse)
 
+// GATED: the tile's 128 columns of the gate AND of the linear branch (rows n_out further on in W): every wavefront holds four
+// accumulators, the A fragments serve both products, and the epilogue stores the gated unit.
+template <bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Wt, int mode, int K, int n_out,
                                                              int top, const int32_t *__restrict__ perm, const int32_t *__restrict__ offsets,
                                                              const int32_t *__restrict__ tile_expert, const int32_t *__restrict__ tile_row0,
-                                                             const float *__restrict__ weights, void *__restrict__ out) {
+                                                             const float *__restrict__ weights, void *__restrict__ out, MoeAct act) {
     __shared__ __attribute__((aligned(16))) bf16_t As[MOE_TM * MM_LD];
-    __shared__ __attribute__((aligned(16))) bf16_t Bs[MM_TN * MM_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[(GATED ? 2 : 1) * MM_TN * MM_LD];
     __shared__ int rin[MOE_TM];
     const int e = tile_expert[blockIdx.x];
     if (e < 0) return;
@@ -196,21 +211,22 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     if (tid < MOE_TM) rin[tid] = tid < nr ? (mode != 1 ? perm[r0 + tid] / top : r0 + tid) : -1;
     __syncthreads();
-    const bf16_t *We = Wt + (int64_t)e * n_out * K;
-    // loaders: 8 bf16 (16 bytes) per thread and row segment; A 64 x 32 = 256 segments, B 128 x 32 = 512 segments
+    const bf16_t *We = Wt + (int64_t)e * (GATED ? 2 : 1) * n_out * K;
+    // loaders: 8 bf16 (16 bytes) per thread and row segment; A 64 x 32 = 256 segments, B 128 x 32 = 512 segments (twice that when GATED)
     const int a_row = tid >> 2, a_seg = (tid & 3) * 8;
     const int64_t a_src = rin[a_row] >= 0 ? (int64_t)rin[a_row] * K : -1;
-    f32x16_t acc0 = {0}, acc1 = {0};
+    f32x16_t acc0 = {0}, acc1 = {0}, acu0 = {0}, acu1 = {0};
     // a stage's rows travel from memory while the previous stage is multiplied: loaded into registers one iteration ahead
-    uint4 av, bv[2];
+    constexpr int NB = GATED ? 4 : 2;
+    uint4 av, bv[NB];
     auto fetch = [&](int k0) {
         av = make_uint4(0, 0, 0, 0);
         if (a_src >= 0 && k0 + a_seg < K) av = *(const uint4 *)(X + a_src + k0 + a_seg);
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int n = (tid >> 2) + 64 * i;
+        for (int i = 0; i < NB; ++i) {
+            const int n = (tid >> 2) + 64 * (i & 1);
             bv[i] = make_uint4(0, 0, 0, 0);
-            if (n0 + n < n_out && k0 + a_seg < K) bv[i] = *(const uint4 *)(We + (int64_t)(n0 + n) * K + k0 + a_seg);
+            if (n0 + n < n_out && k0 + a_seg < K) bv[i] = *(const uint4 *)(We + (int64_t)((i >> 1) * n_out + n0 + n) * K + k0 + a_seg);
         }
     };
     fetch(0);
@@ -222,8 +238,8 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
             d[1] = make_uint2(av.z, av.w);
         }
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            uint2 *d = (uint2 *)(Bs + ((tid >> 2) + 64 * i) * MM_LD + a_seg);
+        for (int i = 0; i < NB; ++i) {
+            uint2 *d = (uint2 *)(Bs + ((tid >> 2) + 64 * i) * MM_LD + a_seg);     // rows 0-127: gate (or the only) columns, 128-255: linear branch
             d[0] = make_uint2(bv[i].x, bv[i].y);
             d[1] = make_uint2(bv[i].z, bv[i].w);
         }
@@ -237,6 +253,11 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
             const bf16x4_t a1 = *(const bf16x4_t *)(As + (32 + (lane & 31)) * MM_LD + ko);
             acc0 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a0, b, acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a1, b, acc1, 0, 0, 0);
+            if (GATED) {
+                const bf16x4_t bu = *(const bf16x4_t *)(Bs + (MM_TN + wave * 32 + (lane & 31)) * MM_LD + ko);
+                acu0 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a0, bu, acu0, 0, 0, 0);
+                acu1 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a1, bu, acu1, 0, 0, 0);
+            }
         }
     }
     const int n = n0 + wave * 32 + (lane & 31);
@@ -249,7 +270,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
             if (m >= nr) continue;
             const float c = half ? acc1[i] : acc0[i];
             const int r = r0 + m;
-            if (mode == JL_MOE_UP_PLAIN) {
+            if (GATED) {
+                st_f((bf16_t *)out + (int64_t)r * n_out + n, gated_unit_f(c, half ? acu1[i] : acu0[i], act.kind, act.limit, act.alpha, act.shift));
+            } else if (mode == JL_MOE_UP_PLAIN) {
                 st_f((bf16_t *)out + (int64_t)r * n_out + n, c);
             } else if (mode == 0) {
                 const float v = fmaxf(c, 0.f);
@@ -261,6 +284,31 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
         }
 }
 
+static int moe_gemm_launch(const void *X, const void *Wt, int dtype, int32_t mode, int32_t K, int32_t n_out, int32_t top, const int32_t *perm,
+                           const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0, int32_t max_tiles, const float *weights,
+                           void *out, const MoeAct *act, void *stream) {
+    static const bool no_mfma = getenv("JL_MOE_NO_MFMA") != nullptr;      // A/B switch for measurements
+    const MoeAct none = {0, 0.f, 0.f, 0.f};
+    if (!no_mfma && dtype == JL_BF16 && K % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0) {
+        const dim3 mgrid((unsigned)max_tiles, (unsigned)((n_out + MM_TN - 1) / MM_TN));
+        if (act)
+            moe_gemm_mfma_kernel<true><<<mgrid, 256, 0, (hipStream_t)stream>>>((const bf16_t *)X, (const bf16_t *)Wt, mode, K, n_out, top, perm, offsets,
+                                                                              tile_expert, tile_row0, weights, out, *act);
+        else
+            moe_gemm_mfma_kernel<false><<<mgrid, 256, 0, (hipStream_t)stream>>>((const bf16_t *)X, (const bf16_t *)Wt, mode, K, n_out, top, perm, offsets,
+                                                                               tile_expert, tile_row0, weights, out, none);
+        return jl_check_launch("moe_gemm_mfma_kernel");
+    }
+    const dim3 grid((unsigned)max_tiles, (unsigned)((n_out + MOE_TN - 1) / MOE_TN));
+    if (act)
+        JL_DISPATCH(dtype, moe_gemm_kernel<T, true><<<grid, 256, 0, (hipStream_t)stream>>>((const T *)X, (const T *)Wt, mode, K, n_out, top, perm, offsets,
+                                                                                           tile_expert, tile_row0, weights, out, *act));
+    else
+        JL_DISPATCH(dtype, moe_gemm_kernel<T, false><<<grid, 256, 0, (hipStream_t)stream>>>((const T *)X, (const T *)Wt, mode, K, n_out, top, perm, offsets,
+                                                                                            tile_expert, tile_row0, weights, out, none));
+    return jl_check_launch("moe_gemm_kernel");
+}
+
 extern "C" int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mode, int32_t K, int32_t n_out, int32_t top,
                            const int32_t *perm, const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0,
                            int32_t max_tiles, const float *weights, void *out, void *stream) {
@@ -268,15 +316,16 @@ extern "C" int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mod
     if (!X || !Wt || !perm || !offsets || !tile_expert || !tile_row0 || !out || (mode == 1 && !weights))
         return jl_fail(JL_E_INVALID, "jl_moe_gemm: null pointer");
     if (K <= 0 || n_out <= 0 || top <= 0 || (mode != 0 && mode != 1 && mode != JL_MOE_UP_PLAIN)) return jl_fail(JL_E_INVALID, "jl_moe_gemm: bad sizes or mode");
-    static const bool no_mfma = getenv("JL_MOE_NO_MFMA") != nullptr;      // A/B switch for measurements
-    if (!no_mfma && dtype == JL_BF16 && K % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0) {
-        const dim3 mgrid((unsigned)max_tiles, (unsigned)((n_out + MM_TN - 1) / MM_TN));
-        moe_gemm_mfma_kernel<<<mgrid, 256, 0, (hipStream_t)stream>>>((const bf16_t *)X, (const bf16_t *)Wt, mode, K, n_out, top, perm, offsets,
-                                                                    tile_expert, tile_row0, weights, out);
-        return jl_check_launch("moe_gemm_mfma_kernel");
-    }
-    const dim3 grid((unsigned)max_tiles, (unsigned)((n_out + MOE_TN - 1) / MOE_TN));
-    JL_DISPATCH(dtype, moe_gemm_kernel<T><<<grid, 256, 0, (hipStream_t)stream>>>((const T *)X, (const T *)Wt, mode, K, n_out, top, perm, offsets,
-                                                                                 tile_expert, tile_row0, weights, out));
-    return jl_check_launch("moe_gemm_kernel");
+    return moe_gemm_launch(X, Wt, dtype, mode, K, n_out, top, perm, offsets, tile_expert, tile_row0, max_tiles, weights, out, nullptr, stream);
+}
+
+extern "C" int jl_moe_gemm_gated(const void *X, const void *Wt, int dtype, int32_t K, int32_t ff, int32_t top, const int32_t *perm,
+                                 const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0, int32_t max_tiles, int32_t kind,
+                                 float limit, float alpha, float shift, void *out, void *stream) {
+    if (max_tiles <= 0) return JL_OK;
+    if (!X || !Wt || !perm || !offsets || !tile_expert || !tile_row0 || !out) return jl_fail(JL_E_INVALID, "jl_moe_gemm_gated: null pointer");
+    if (K <= 0 || ff <= 0 || top <= 0 || (kind != JL_ACT_GELU_TANH && kind != JL_ACT_CLAMPED_SWISH))
+        return jl_fail(JL_E_INVALID, "jl_moe_gemm_gated: bad sizes or kind");
+    const MoeAct act = {kind, limit, alpha, shift};
+    return moe_gemm_launch(X, Wt, dtype, JL_MOE_UP_PLAIN, K, ff, top, perm, offsets, tile_expert, tile_row0, max_tiles, nullptr, out, &act, stream);
 }

@@ -106,9 +106,6 @@ extern "C" int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n
 }
 
 // ---- gated activation of a feed-forward: out[n, c] = act(z[n, g_col + c]) * lin(z[n, u_col + c]) (* sigmoid(row_gate[n])) -----------------
-__device__ __forceinline__ float gelu_tanh_f(float z) {
-    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-}
 template <typename T>
 __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ z, int64_t ld, int g_col, int u_col, int F, int kind, float limit, float alpha,
                                                          float shift, const T *__restrict__ row_gate, int64_t rg_ld, T *__restrict__ out, int64_t total) {
@@ -116,16 +113,47 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ z,
     if (e >= total) return;
     const int64_t n = e / F;
     const int c = (int)(e - n * F);
-    float g = ld_f(z + n * ld + g_col + c), u = ld_f(z + n * ld + u_col + c), v;
-    if (kind == JL_ACT_GELU_TANH) {
-        v = gelu_tanh_f(g) * u;
-    } else {                                                        // clamped swish: the gate capped from above, the linear branch from both sides
-        g = fminf(g, limit);
-        u = fminf(fmaxf(u, -limit), limit);
-        v = g / (1.0f + expf(-alpha * g)) * (u + shift);
-    }
+    float v = gated_unit_f(ld_f(z + n * ld + g_col + c), ld_f(z + n * ld + u_col + c), kind, limit, alpha, shift);
     if (row_gate) v *= 1.0f / (1.0f + expf(-ld_f(row_gate + n * rg_ld)));
     st_f(out + e, v);
+}
+
+// 16 bytes per load and thread (4 floats, 8 bfloat16): columns, row stride and F in multiples of that
+__device__ __forceinline__ void ld16(const float *p, float (&v)[4]) { const float4 t = *(const float4 *)p; v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+__device__ __forceinline__ void ld16(const bf16_t *p, float (&v)[8]) {
+    const uint4 t = *(const uint4 *)p;
+    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(w[i] << 16); v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+}
+__device__ __forceinline__ void st16(float *p, const float (&v)[4]) { *(float4 *)p = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void st16(bf16_t *p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        bf16_t lo, hi;
+        st_f(&lo, v[2 * i]);
+        st_f(&hi, v[2 * i + 1]);
+        w[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+    *(uint4 *)p = make_uint4(w[0], w[1], w[2], w[3]);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void gated_act_vec_kernel(const T *__restrict__ z, int64_t ld, int g_col, int u_col, int F, int kind, float limit, float alpha,
+                                                             float shift, const T *__restrict__ row_gate, int64_t rg_ld, T *__restrict__ out, int64_t vecs) {
+    constexpr int VEC = 16 / sizeof(T);
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= vecs) return;
+    const int per_row = F / VEC;
+    const int64_t n = e / per_row;
+    const int c = (int)(e - n * per_row) * VEC;
+    float g[VEC], u[VEC];
+    ld16(z + n * ld + g_col + c, g);
+    ld16(z + n * ld + u_col + c, u);
+    const float rg = row_gate ? 1.0f / (1.0f + expf(-ld_f(row_gate + n * rg_ld))) : 1.0f;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) g[i] = gated_unit_f(g[i], u[i], kind, limit, alpha, shift) * rg;
+    st16(out + n * F + c, g);
 }
 
 extern "C" int jl_gated_act(const void *z, int dtype, int64_t N, int64_t ld, int32_t g_col, int32_t u_col, int32_t F, int32_t kind, float limit, float alpha,
@@ -134,6 +162,13 @@ extern "C" int jl_gated_act(const void *z, int dtype, int64_t N, int64_t ld, int
     if (!z || !out || F <= 0 || g_col < 0 || u_col < 0 || g_col + (int64_t)F > ld || u_col + (int64_t)F > ld)
         return jl_fail(JL_E_INVALID, "jl_gated_act: null pointer, or the columns do not fit the row stride");
     if (kind != JL_ACT_GELU_TANH && kind != JL_ACT_CLAMPED_SWISH) return jl_fail(JL_E_INVALID, "jl_gated_act: unknown kind %d", kind);
+    const int vec = dtype == JL_BF16 ? 8 : 4;
+    if (F % vec == 0 && g_col % vec == 0 && u_col % vec == 0 && ld % vec == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
+        const int64_t vecs = N * (F / vec);
+        JL_DISPATCH(dtype, gated_act_vec_kernel<T><<<dim3((unsigned)((vecs + 255) / 256)), 256, 0, (hipStream_t)stream>>>(
+                               (const T *)z, ld, g_col, u_col, F, kind, limit, alpha, shift, (const T *)row_gate, rg_ld, (T *)out, vecs));
+        return jl_check_launch("gated_act_vec_kernel");
+    }
     const int64_t total = N * F;
     JL_DISPATCH(dtype, gated_act_kernel<T><<<dim3((unsigned)((total + 255) / 256)), 256, 0, (hipStream_t)stream>>>(
                            (const T *)z, ld, g_col, u_col, F, kind, limit, alpha, shift, (const T *)row_gate, rg_ld, (T *)out, total));

@@ -1,9 +1,9 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of a ragged model family (Lokizen, Vumalix) at sizes that resemble a real model's layers, beside
-the package's closest existing model at equal width, depth, head sizes and active feed-forward width (Lokizen beside Qwen2;
-Vumalix beside Lokizen and Qwen2) — random weights, synthetic tokens.
+"""Prefill and decode throughput of a ragged model family (Lokizen, Vumalix, Bamanex) at sizes that resemble a real model's layers,
+beside the package's closest existing model at equal width, depth, head sizes and active feed-forward width (Lokizen beside Qwen2;
+Vumalix beside Lokizen and Qwen2; Bamanex beside Lokizen and Qwen2) — random weights, synthetic tokens.
 
-    python -m jacobiforcing_amd.drivers.ragged_bench [--design lokizen|vumalix] [--sizes small,medium] [--kernels]
+    python -m jacobiforcing_amd.drivers.ragged_bench [--design lokizen|vumalix|bamanex] [--sizes small,medium] [--kernels]
     python bench.py --design lokizen            (the same, as one JSON line)
 
 Per size: prefill = whole prompts in one step (tokens / s), decode = one token for each of ``--decode-batch`` requests at a
@@ -300,6 +300,121 @@ def kernel_table_vumalix(s, prompts, prompt_len, decode_batch, context, dtype=to
 SIZES_BY_WIDTH = {v["width"]: v for v in SIZES.values()}
 
 
+# Bamanex at Lokizen's widths, depths, head counts and windows: every layer is attention; dense feed-forwards (of the experts' active
+# width) and expert feed-forwards (Lokizen's expert count, choice size and width, plus a shared expert) alternate
+def bamanex_config(s):
+    from ..modeling.bamanex import BamanexConfig
+    H, D = s["heads"], s["dim"]
+    mixer = {"heads": H, "kv_heads": s["kv"], "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": s["window"]},
+             "rot": {"dims": D // 2, "base": 1e6, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    moe = {"kind": "moe", "expert": {"ff": s["ff"], "limit": 7.0}, "router": {"experts": s["experts"], "top": s["top"]}, "shared": {"ff": s["ff"], "limit": 7.0}}
+    dense = {"kind": "dense", "ff": s["top"] * s["ff"]}
+    return BamanexConfig.from_dict({"architecture": "Bamanex", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+                                    "layers": [{"type": "attention", "mixer": mixer, "mlp": dense if i % 2 == 0 else moe} for i in range(s["layers"])]})
+
+
+def bench_bamanex(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
+    from ..modeling.bamanex import random_model
+    model = random_model(bamanex_config(s), "cuda", dtype, max_positions=max(prompt_len, context) + 64)
+    return bench_ragged(model, s["vocab"], prompts, prompt_len, decode_batch, context)
+
+
+def kernel_table_bamanex(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
+    """Bamanex's layer kernels alone at the size's shapes, prefill and decode, each beside the like kernel of the closest model
+    (Lokizen's residual + norm launch, its whole-projection q/k norm, its windowed attention, its routed experts; Qwen2's SwiGLU
+    launch)."""
+    from .. import layer_ops as LO
+    from .. import ops
+    dev = "cuda"
+    H, G, D, W, E, top, ff, win = s["heads"], s["kv"], s["dim"], s["width"], s["experts"], s["top"], s["ff"], s["window"]
+    page, es = 64, 2
+    per = -(-(max(prompt_len, context) + 1) // page)
+    slots = max(prompts, decode_batch)
+    tables = [list(range(b * per, (b + 1) * per)) for b in range(slots)]
+    g = torch.Generator().manual_seed(0)
+    rnd = lambda *sh: torch.randn(*sh, generator=g).to(dev).to(dtype)
+    kc, vc = rnd(slots * per * page, G * D), rnd(slots * per * page, G * D)
+    rd = D // 2
+    a = torch.arange(max(prompt_len, context) + 8, dtype=torch.float32, device=dev).view(-1, 1) * torch.rand(rd // 2, device=dev).view(1, -1)
+    cos, sin = a.cos().contiguous(), a.sin().contiguous()
+    sink = torch.randn(H, device=dev)
+    w_gu, w_up, w_down = rnd(E, 2 * ff, W) * 0.02, rnd(E, ff, W) * 0.02, rnd(E, W, ff) * 0.02
+    out = {}
+
+    def row(name, secs, nbytes, flops, peak):
+        bound = max(nbytes / HBM_BPS, flops / peak)
+        out[name] = {"us": round(1e6 * secs, 1), "MB": round(nbytes / 1e6, 2), "GFLOP": round(flops / 1e9, 2), "roofline_fraction": round(bound / secs, 4)}
+
+    for phase, B, T, start in (("prefill", prompts, prompt_len, 0), ("decode", decode_batch, 1, context)):
+        n = B * T
+        batch = LO.RaggedBatch.build([T] * B, [start] * B, list(range(B)), tables[:B], page, dev)
+        windowed = B * sum(min(start + t + 1, win) for t in range(T))                              # visible (query, key) pairs per head
+        span_w = B * min(start + T, win + T)                                                       # pool rows a launch has to read once
+        # residual sum of two scaled sublayer outputs + both norms  |  Lokizen: one addend, one norm
+        x, y1, y2, wn = torch.randn(n, W, device=dev), rnd(n, W), rnd(n, W), rnd(W)
+        ls, w1 = torch.rand(W, device=dev), torch.randn(W, device=dev) * 0.1
+        row(f"{phase}.scaled_add_norms", timed(lambda: LO.scaled_add_norms(x, [(y1, ls), (y2, ls)], w1, w1, 1.0, 1e-6, dtype, two=True)),
+            n * W * (4 + 4 + 4 * es), 8.0 * n * W, VECTOR_FLOPS)
+        row(f"{phase}.lokizen.add_rmsnorm", timed(lambda: LO.add_rmsnorm(x, y1, None, wn, 1e-5, dtype)), n * W * (4 + 4 + es + es), 4.0 * n * W, VECTOR_FLOPS)
+        # rotation + per-head unit norm + append  |  Lokizen: whole-projection norm + append
+        proj = rnd(n, H * D + 2 * G * D + H)
+        cols = (0, H * D, H * D + G * D)
+        t_hn = timed(lambda: LO.head_norm_append(proj, cols, H, G, 1, D, D, None, None, 1e-6, 0.0, 1, batch, kc, vc, rot_dims=rd, cos=cos, sin=sin))
+        row(f"{phase}.head_norm_append(rot)", t_hn, 2 * n * (H * D + 2 * G * D) * es, 10.0 * n * (H + G) * D, VECTOR_FLOPS)
+        pk = rnd(n, H * D + 2 * G * D)
+        wqk, wkk = rnd(H * D), rnd(G * D)
+        t_qk = timed(lambda: LO.qk_norm_append(pk, cols, H, G, D, D, wqk, wkk, 1e-5, kc, vc, batch.kv_slot))
+        row(f"{phase}.lokizen.qk_norm_append", t_qk, 2 * n * (H * D + 2 * G * D) * es, 6.0 * n * (H + G) * D, VECTOR_FLOPS)
+        # attention with sink and head gate  |  Lokizen: window keeping first tokens, distance bias, mixed heads, element gate
+        q = LO.head_norm_append(proj, cols, H, G, 1, D, D, None, None, 1e-6, 0.0, 1, batch, kc, vc, rot_dims=rd, cos=cos, sin=sin)
+        hg = proj[:, H * D + 2 * G * D:]
+        sweep = LO.attn_sweep_tile_rows(dtype, H, G, D, D, kc, vc) > 0
+
+        def sink_attn():
+            if sweep:
+                return LO.attn_sweep(q, kc, vc, batch, H, G, D, D, D ** -0.5, win, sink=sink, gate=hg, gate_per_head=True)
+            return LO.attn_window(q, hg, kc, vc, batch, H, G, D, D, D ** -0.5, win, 0, None, None, None, sink=sink, gate_per_head=True)
+        row(f"{phase}.attn_sink_gate", timed(sink_attn), span_w * 2 * G * D * es + 2 * n * H * D * es, 4.0 * windowed * H * D, MATRIX_FLOPS)
+        gate = rnd(n, H * D)
+        rel, talk = torch.randn(max(prompt_len, context) + 8, H, device=dev), torch.eye(H, device=dev)
+        t_att = timed(lambda: LO.attn_window(q, gate, kc, vc, batch, H, G, D, D, D ** -0.5, win, 4, rel, None, talk))
+        row(f"{phase}.lokizen.attn_window", t_att, span_w * 2 * G * D * es + 3 * n * H * D * es, 4.0 * windowed * H * D, MATRIX_FLOPS)
+        # gated activations  |  Qwen2's SwiGLU launch
+        gu = rnd(n, 2 * top * ff)
+        row(f"{phase}.gated_act(gelu)", timed(lambda: LO.gated_act(gu, 0, top * ff, top * ff, LO.ACT_GELU_TANH)), 3 * n * top * ff * es, 12.0 * n * top * ff, VECTOR_FLOPS)
+        gs = rnd(n, 2 * ff + 8)                                # gate, linear branch, the token gate, zero columns up to a 16-byte border
+        row(f"{phase}.gated_act(clamped, row gate)", timed(lambda: LO.gated_act(gs, 0, ff, ff, LO.ACT_CLAMPED_SWISH, 7.0, 1.702, 1.0, row_gate=gs[:, 2 * ff])),
+            3 * n * ff * es, 10.0 * n * ff, VECTOR_FLOPS)
+        row(f"{phase}.qwen2.swiglu", timed(lambda: ops.swiglu(gu)), 3 * n * top * ff * es, 4.0 * n * top * ff, VECTOR_FLOPS)
+        # routed experts: clamped gated units, softmax routing  |  Lokizen: relu^2 units, sigmoid routing
+        h, z = rnd(n, W), torch.randn(n, E, device=dev)
+        used = min(E, n * top)
+        t_moe = timed(lambda: LO.moe_experts(h, z, None, top, 1.0, w_gu, w_down, route="softmax_renorm", renorm_eps=1e-20,
+                                             gated=(LO.ACT_CLAMPED_SWISH, 7.0, 1.702, 1.0)))
+        row(f"{phase}.moe_experts(gated)", t_moe, used * 3 * ff * W * es + n * W * es + n * top * W * 4, 6.0 * n * top * ff * W, MATRIX_FLOPS)
+        t_moe = timed(lambda: LO.moe_experts(h, z, None, top, 1.0, w_up, w_down))
+        row(f"{phase}.lokizen.moe_experts", t_moe, used * 2 * ff * W * es + n * W * es + n * top * W * 4, 4.0 * n * top * ff * W, MATRIX_FLOPS)
+    return out
+
+
+def run_bamanex(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True):
+    res = {"bench": "ragged_family", "design": "Bamanex", "closest": "Lokizen", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
+           "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
+    for name in sizes:
+        s = SIZES[name]
+        entry = {"shape": s, "bamanex": bench_bamanex(s, prompts, prompt_len, decode_batch, context)}
+        torch.cuda.empty_cache()
+        entry["lokizen"] = bench_lokizen(s, prompts, prompt_len, decode_batch, context)
+        torch.cuda.empty_cache()
+        entry["qwen2"] = bench_qwen2(s, prompts, prompt_len, decode_batch, context)
+        torch.cuda.empty_cache()
+        if kernels:
+            entry["kernels"] = kernel_table_bamanex(s, prompts, prompt_len, decode_batch, context)
+            torch.cuda.empty_cache()
+        res["sizes"][name] = entry
+    return res
+
+
 def run_vumalix(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True):
     res = {"bench": "ragged_family", "design": "Vumalix", "closest": "Lokizen", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
            "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
@@ -321,6 +436,8 @@ def run_vumalix(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_ba
 def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True, design="lokizen"):
     if design.lower() == "vumalix":
         return run_vumalix(sizes, prompts, prompt_len, decode_batch, context, kernels)
+    if design.lower() == "bamanex":
+        return run_bamanex(sizes, prompts, prompt_len, decode_batch, context, kernels)
     res = {"bench": "ragged_family", "design": "Lokizen", "closest": "Qwen2", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
            "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
     for name in sizes:
@@ -338,7 +455,7 @@ def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
-    ap.add_argument("--design", default="lokizen", choices=("lokizen", "vumalix"))
+    ap.add_argument("--design", default="lokizen", choices=("lokizen", "vumalix", "bamanex"))
     ap.add_argument("--sizes", default="small,medium")
     ap.add_argument("--prompts", type=int, default=4)
     ap.add_argument("--prompt-len", type=int, default=2048)

@@ -333,7 +333,7 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
     ``route`` "sigmoid": sigmoid scores, choice by score + correction, weights = score * scale; "softmax_renorm": softmax over all
     experts, the largest chosen, weights = score / (sum of the chosen + renorm_eps) * scale.
     ``gated`` None: experts down(relu(up h)^2) with w_up [E, ff, W].  ``gated`` = (kind, limit, alpha, shift) of ``gated_act``: w_up
-    [E, 2*ff, W] stacks every expert's gate rows on its linear rows, and the activation is a launch between the two products."""
+    [E, 2*ff, W] stacks every expert's gate rows on its linear rows, and the up product applies the unit in its epilogue."""
     _dev(h)
     n, W = h.shape
     E, ff = w_down.shape[0], w_down.shape[2]
@@ -359,11 +359,16 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
     tile_e = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
     tile_r = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
     N.check_layers(L.jl_moe_group(_ptr(ids), n, top, E, tm, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles, st), "jl_moe_group")
-    act = torch.empty((rows, up_rows), dtype=dt, device=dev)
-    N.check_layers(L.jl_moe_gemm(_ptr(h), _ptr(w_up), _code(dt), N.JL_MOE_UP_PLAIN if gated is not None else N.JL_MOE_UP_RELU2, W, up_rows, top, _ptr(perm),
-                                 _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles, None, _ptr(act), st), "jl_moe_gemm(up)")
-    if gated is not None:
-        act = gated_act(act, 0, ff, ff, *gated)
+    if gated is not None and not os.environ.get("JL_MOE_UNFUSED_ACT"):          # the unit in the product's epilogue (A/B switch for measurements)
+        act = torch.empty((rows, ff), dtype=dt, device=dev)
+        N.check_layers(L.jl_moe_gemm_gated(_ptr(h), _ptr(w_up), _code(dt), W, ff, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
+                                           int(gated[0]), float(gated[1]), float(gated[2]), float(gated[3]), _ptr(act), st), "jl_moe_gemm_gated")
+    else:
+        act = torch.empty((rows, up_rows), dtype=dt, device=dev)
+        N.check_layers(L.jl_moe_gemm(_ptr(h), _ptr(w_up), _code(dt), N.JL_MOE_UP_PLAIN if gated is not None else N.JL_MOE_UP_RELU2, W, up_rows, top, _ptr(perm),
+                                     _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles, None, _ptr(act), st), "jl_moe_gemm(up)")
+        if gated is not None:
+            act = gated_act(act, 0, ff, ff, *gated)
     y = torch.empty((n, top, W), dtype=torch.float32, device=dev)
     N.check_layers(L.jl_moe_gemm(_ptr(act), _ptr(w_down), _code(dt), N.JL_MOE_DOWN, ff, W, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
                                  _ptr(wts), _ptr(y), st), "jl_moe_gemm(down)")

@@ -130,14 +130,17 @@ class BamanexWeights:
         if tuple(self.embed.shape) != (cfg.vocab_size, W):
             raise ValueError(f"embed is {tuple(self.embed.shape)}, config says {(cfg.vocab_size, W)}")
         self.layers = []
+        # a stacked matrix ends with zero rows up to a multiple of eight: the product's rows then start at 16-byte borders
+        pad = lambda rows: torch.zeros(((-rows) % 8, W), dtype=dtype, device=dev)
         for i, L in enumerate(cfg.layers):
             p, m = f"l{i}.", L["mixer"]
             H, G, D, Dv = (int(m[k]) for k in ("heads", "kv_heads", "dim", "vdim"))
+            rows = H * D + G * D + G * Dv + H
             w = dict(norm1=f32(p + "norm1"), ls1=f32(p + "ls1"), sink=f32(p + "mix.sink"), w_o=act(p + "mix.o"), b_o=act(p + "mix.o.b"),
-                     w_in=torch.cat([act(p + "mix.q"), act(p + "mix.k"), act(p + "mix.v"), act(p + "mix.g")], 0),
-                     b_in=torch.cat([act(p + "mix.q.b"), act(p + "mix.k.b"), act(p + "mix.v.b"), torch.zeros(H, dtype=dtype, device=dev)], 0),
+                     w_in=torch.cat([act(p + "mix.q"), act(p + "mix.k"), act(p + "mix.v"), act(p + "mix.g"), pad(rows)], 0),
+                     b_in=torch.cat([act(p + "mix.q.b"), act(p + "mix.k.b"), act(p + "mix.v.b"), torch.zeros(H + (-rows) % 8, dtype=dtype, device=dev)], 0),
                      cols=(0, H * D, H * D + G * D, H * D + G * D + G * Dv))
-            if w["w_in"].shape[0] != H * D + G * D + G * Dv + H or w["sink"].numel() != H or tuple(w["w_o"].shape) != (W, H * Dv):
+            if w["w_in"].shape[0] != rows + (-rows) % 8 or w["sink"].numel() != H or tuple(w["w_o"].shape) != (W, H * Dv):
                 raise ValueError(f"layer {i}: the mixer's tensors do not fit heads={H} kv_heads={G} dim={D} vdim={Dv}")
             f = L.get("mlp")
             if f is not None:
@@ -154,10 +157,11 @@ class BamanexWeights:
                     if tuple(w["w_gu"].shape) != (E, 2 * ff, W) or tuple(w["router"].shape) != (E, W):
                         raise ValueError(f"layer {i}: experts are {tuple(w['w_gu'].shape)}, config says {E} experts of ff {ff}")
                     if f.get("shared") is not None:
-                        w.update(w_sh=torch.cat([act(p + "mlp.shared.gate"), act(p + "mlp.shared.up"), act(p + "mlp.shared.sg").view(1, W)], 0),
+                        fs = int(f["shared"]["ff"])
+                        w.update(w_sh=torch.cat([act(p + "mlp.shared.gate"), act(p + "mlp.shared.up"), act(p + "mlp.shared.sg").view(1, W), pad(2 * fs + 1)], 0),
                                  w_sh_down=act(p + "mlp.shared.down"))
-                        if w["w_sh"].shape[0] != 2 * int(f["shared"]["ff"]) + 1:
-                            raise ValueError(f"layer {i}: the shared expert has {w['w_sh'].shape[0] - 1} gate / up rows, config says ff {f['shared']['ff']}")
+                        if w["w_sh"].shape[0] != 2 * fs + 1 + (-(2 * fs + 1)) % 8:
+                            raise ValueError(f"layer {i}: the shared expert's gate / up do not have the {fs} rows each that the config says")
             self.layers.append(w)
 
     @classmethod

@@ -91,6 +91,15 @@ def rel_err(got, want):
 F32_TOL, BF16_TOL = 2e-4, 6e-2
 
 
+def rows_off(got, want, tol):
+    """Fraction of rows (positions) whose own relative error is above ``tol``.  In bfloat16 a router's close call may go the other
+    way for a token or two — such a token's row is simply another expert's, by much more than rounding — so a test over random
+    routers bounds how many rows differ instead of their common error."""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    err = np.sqrt(((got - want) ** 2).mean(-1)) / np.maximum(np.sqrt((want ** 2).mean(-1)), 1e-30)
+    return float((err > tol).mean())
+
+
 def toks(n, vocab, seed):
     return [random.Random(seed * 7919 + i).randrange(vocab) for i in range(n)]
 
@@ -124,8 +133,10 @@ def test_one_pool_per_layer_run_and_stacked_weights():
     specs = BX.BamanexModel(cfg, w, max_positions=16).cache_specs()
     assert len(specs) == 8 and [(s.k_width, s.v_width) for s in specs[:3]] == [(48, 80), (64, 64), (32, 24)] and specs[3].k_width == 64
     l0, l1, l3 = w.layers[0], w.layers[1], w.layers[3]
-    assert tuple(l0["w_in"].shape) == (6 * 24 + 2 * 24 + 2 * 40 + 6, 96) and l0["cols"] == (0, 144, 192, 272) and float(l0["b_in"][-6:].abs().sum()) == 0
-    assert tuple(l0["w_gu"].shape) == (112, 96) and tuple(l1["w_gu"].shape) == (5, 48, 96) and tuple(l1["w_sh"].shape) == (81, 96)
+    # q, k, v and the six head gates, then zero rows up to a multiple of eight (the gates and the padding have no bias)
+    assert tuple(l0["w_in"].shape) == (6 * 24 + 2 * 24 + 2 * 40 + 6 + 2, 96) and l0["cols"] == (0, 144, 192, 272) and float(l0["b_in"][-8:].abs().sum()) == 0
+    assert float(l0["w_in"][-2:].abs().sum()) == 0 and float(l0["w_in"][-8:-2].abs().sum()) > 0
+    assert tuple(l0["w_gu"].shape) == (112, 96) and tuple(l1["w_gu"].shape) == (5, 48, 96) and tuple(l1["w_sh"].shape) == (88, 96)
     assert "w_sh" not in l3 and "norm2" not in w.layers[2] and l0["norm1"].dtype == torch.float32 and l1["router"].dtype == torch.float32
 
 
@@ -265,7 +276,7 @@ def test_gated_activations(F_):
 
 @gpu
 @pytest.mark.parametrize("E,top,ff,W", [(5, 2, 24, 96), (3, 1, 20, 64), (4, 4, 33, 50), (16, 3, 64, 128)])
-def test_softmax_router_and_clamped_experts_alone(E, top, ff, W):
+def test_softmax_router_and_clamped_experts_alone(E, top, ff, W, monkeypatch):
     from jacobiforcing_amd import layer_ops as LO
     cfg = make_cfg([dict(attn(), mlp=moe(experts=E, top=top, ff=ff, limit=1.25, shared_ff=0))], width=W)
     t = tensors_for(cfg, E)
@@ -277,11 +288,14 @@ def test_softmax_router_and_clamped_experts_alone(E, top, ff, W):
     for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
         w = BX.BamanexWeights(BX.BamanexConfig.from_dict(cfg), t, "cuda", dtype).layers[0]
         hd = h.cuda().to(dtype)
-        y = LO.moe_experts(hd, torch.nn.functional.linear(hd.float(), w["router"]), None, top, 1.0, w["w_gu"], w["w_down"], route="softmax_renorm",
-                           renorm_eps=1e-20, gated=(LO.ACT_CLAMPED_SWISH, 1.25, 1.702, 1.0))
-        assert tuple(y.shape) == (70, top, W) and y.dtype == torch.float32
         ref = want if dtype == torch.float32 else O.expert_mixture(h.bfloat16().double(), P, f)
-        assert rel_err(y.sum(1).cpu(), ref) < tol, dtype
+        for unfused in ("", "1"):                         # the unit in the up product's epilogue, and as a launch of its own
+            monkeypatch.setenv("JL_MOE_UNFUSED_ACT", unfused)
+            y = LO.moe_experts(hd, torch.nn.functional.linear(hd.float(), w["router"]), None, top, 1.0, w["w_gu"], w["w_down"], route="softmax_renorm",
+                               renorm_eps=1e-20, gated=(LO.ACT_CLAMPED_SWISH, 1.25, 1.702, 1.0))
+            assert tuple(y.shape) == (70, top, W) and y.dtype == torch.float32
+            assert rel_err(y.sum(1).cpu(), ref) < tol, (dtype, unfused)
+        monkeypatch.delenv("JL_MOE_UNFUSED_ACT")
     # ties go to the lower index, and the weights of the chosen sum to one
     z = torch.zeros(2, E)
     z[1, E - 1] = 1.0
@@ -594,7 +608,10 @@ def test_random_configurations_in_a_mixed_schedule(seed):
             out = rig.step(entries)
             got_a.append(out[:na]); got_b.append(out[na:])
             ia += na; ib += nb
-        assert rel_err(torch.cat(got_a), want_a) < tol and rel_err(torch.cat(got_b), want_b) < tol, (seed, dtype, cfg)
+        if dtype == torch.float32:
+            assert rel_err(torch.cat(got_a), want_a) < tol and rel_err(torch.cat(got_b), want_b) < tol, (seed, dtype, cfg)
+        else:
+            assert rows_off(torch.cat(got_a), want_a, tol) <= 0.1 and rows_off(torch.cat(got_b), want_b, tol) <= 0.1, (seed, dtype, cfg)
 
 
 def _write_model(tmp_path, cfg_dict, tensors):
