@@ -386,6 +386,8 @@ def kernel_table_bamanex(s, prompts, prompt_len, decode_batch, context, dtype=to
         row(f"{phase}.gated_act(clamped, row gate)", timed(lambda: LO.gated_act(gs, 0, ff, ff, LO.ACT_CLAMPED_SWISH, 7.0, 1.702, 1.0, row_gate=gs[:, 2 * ff])),
             3 * n * ff * es, 10.0 * n * ff, VECTOR_FLOPS)
         row(f"{phase}.qwen2.swiglu", timed(lambda: ops.swiglu(gu)), 3 * n * top * ff * es, 4.0 * n * top * ff, VECTOR_FLOPS)
+        g1 = rnd(n, 2 * ff)                                    # the same launch at the shared expert's width: the clamped unit's like at equal bytes
+        row(f"{phase}.qwen2.swiglu(shared width)", timed(lambda: ops.swiglu(g1)), 3 * n * ff * es, 4.0 * n * ff, VECTOR_FLOPS)
         # routed experts: clamped gated units, softmax routing  |  Lokizen: relu^2 units, sigmoid routing
         h, z = rnd(n, W), torch.randn(n, E, device=dev)
         used = min(E, n * top)
