@@ -69,8 +69,8 @@ JL_API int jl_qk_norm_append(const void *proj, int dtype, int64_t N, int64_t ld,
  *   s_g(i, j) = q_g(i) . k_c(g)(j) * scale + rel[lut[min(i - j, lut_len - 1)], g]          (c(g) = g / (H / G))
  *   p_g(i, .) = softmax over the visible j;   w_h(i, j) = sum_g talk[h, g] p_g(i, j)  (talk null: w = p)
  *   out_h(i) = (sum_j w_h(i, j) v_c(h)(j)) * sigmoid(gate_h(i))                             (gate null: no gate)
- * With `sink` (float [H], may be null) the softmax's denominator of head g holds one more term exp(sink[g]): a key without a value,
- * neither scaled nor biased, counted once, so the weights of a row sum to less than one.  `gate` is read element by element
+ * With `sink` (float [H], may be null) the softmax's denominator of head g holds one more term exp(sink[g]): an extra
+ * score that attends to nothing (taken as it is: no scale, no bias; present exactly once per row), so a row's weights sum to less than one.  `gate` is read element by element
  * ([N, H*Dv], rows gate_ld apart) or, with gate_heads != 0, one number per head ([N, H], rows gate_ld apart).
  * tiles [n_tiles, 4] int32 = {b, first query position, count (<= TQ), first row}: consecutive rows of one request;
  * block_tables [*, bt_stride] int32 pages of request b in order; a key j lives at token page * page_size + j % page_size of the

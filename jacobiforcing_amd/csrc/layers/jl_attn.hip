@@ -113,7 +113,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
     const T *vc = (const T *)a.v_cache;
 
     for (int e = tid; e < cnt * H * D; e += ATT_THREADS) Qs[e] = ld_f(q + (int64_t)row0 * H * D + e);
-    // a sink is a key without a value: every row starts from its score with a sum of one
+    // a sink acts like one extra score that attends to nothing: every row's statistics start from (sink, 1)
     for (int e = tid; e < H * TQ; e += ATT_THREADS) { mx[e] = a.sink ? a.sink[e / TQ] : -INFINITY; sm[e] = a.sink ? 1.f : 0.f; }
     if (a.talk) for (int e = tid; e < H * H; e += ATT_THREADS) talk[e] = a.talk[e];
 

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(AS_THREADS) void attn_sweep_kernel(jl_attn_args a, 
     const int r_i = i0 + rr / HF;
     const bool r_ok = rr < TQ * HF && rr / HF < cnt && h0 + rr % HF < h_end;
     float m_run = -INFINITY, l_run = 0.f;
-    // a sink is a key without a value, counted once: the row's statistics start from it (in the first share of the keys only)
+    // a sink acts like one extra score that attends to nothing: the row's statistics start from (sink, 1), in the first share of the keys only
     if (a.sink && r_ok && blockIdx.z == 0) { m_run = a.sink[h0 + rr % HF]; l_run = 1.f; }
 
     as_f32x16 acc[NT];

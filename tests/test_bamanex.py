@@ -347,7 +347,7 @@ def test_the_mixer_alone_in_portions_and_single_tokens(H, G, D, Dv, size, dims):
 @gpu
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 1, 64, 64), (8, 2, 32, 96), (6, 2, 24, 40), (3, 3, 20, 12)])
 @pytest.mark.parametrize("size", [0, 300])
-def test_single_tokens_over_a_long_context_count_the_sink_once(H, G, D, Dv, size):
+def test_single_tokens_over_a_long_context_take_the_sink_once(H, G, D, Dv, size):
     """Decoding far into a context shares the keys of a tile out over workgroups; the sink belongs to one share only."""
     cfg = one_layer(H, G, D, Dv, size, 8)
     t = tensors_for(cfg, 3)
