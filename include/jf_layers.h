@@ -41,10 +41,11 @@ JL_API int jl_add_rmsnorm(float *x, const void *y, int y_dtype, int32_t y_count,
  * `w_offset` — the layer whose mixer and feed-forward both read one stream and are added in one sum:
  *   x[n, c] += sum_a scale_a[c] * sum_{s < count_a} y_a[(n * count_a + s), c]        (at most 3 addends; scale null = 1)
  *   out1[n] = x[n] / sqrt(mean(x[n]^2) + eps) * (w_offset + w1);   out2 likewise with w2   (out1 / out2 / w1 / w2 may be null)
- * x float in place; y_a of its own dtype; out1 / out2 of `dtype`. */
+ * x float in place; y_a of its own dtype; out1 / out2 of `dtype`; out2_f32 (may be null) receives the second norm unrounded as well
+ * (what a float router reads beside the bfloat16 copy the experts' products read). */
 typedef struct { const void *y; int32_t dtype; int32_t count; const float *scale; } jl_addend;
 JL_API int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n_addends, const float *w1, const float *w2, float w_offset,
-                               float eps, void *out1, void *out2, int dtype, int64_t N, int32_t W, void *stream);
+                               float eps, void *out1, void *out2, float *out2_f32, int dtype, int64_t N, int32_t W, void *stream);
 
 /* Gated activation of a feed-forward whose gate and linear branch are column ranges of one product z [N, ld] (F columns each at
  * g_col / u_col):   out[n, c] = act(g) * lin(u) * sigmoid(row_gate[n * rg_ld])        (row_gate null: no row gate)

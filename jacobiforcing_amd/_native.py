@@ -270,7 +270,7 @@ _LAYER_SIGNATURES = {
     "jl_causal_conv_carry": (C.c_int, [_vp, _vp, _i32, _vp, _i32, _i32, _vp]),
     "jl_head_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _f32, _i32,
                                       _vp, _vp, _i32, _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
-    "jl_scaled_add_norms": (C.c_int, [_vp, C.POINTER(Addend), _i32, _vp, _vp, _f32, _f32, _vp, _vp, C.c_int, _i64, _i32, _vp]),
+    "jl_scaled_add_norms": (C.c_int, [_vp, C.POINTER(Addend), _i32, _vp, _vp, _f32, _f32, _vp, _vp, _vp, C.c_int, _i64, _i32, _vp]),
     "jl_gated_act": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _f32, _f32, _f32, _vp, _i64, _vp, _vp]),
     "jl_diff_combine": (C.c_int, [_vp, _vp, _i64, _i64, _i32, _i32, _f32, _f32, _f32, _vp, C.c_int, _vp]),
     "jl_latent_prep": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _vp, _vp,

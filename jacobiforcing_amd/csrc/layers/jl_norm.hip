@@ -62,7 +62,7 @@ extern "C" int jl_add_rmsnorm(float *x, const void *y, int y_dtype, int32_t y_co
 template <typename T>
 __global__ __launch_bounds__(256) void scaled_add_norms_kernel(float *__restrict__ x, jl_addend a0, jl_addend a1, jl_addend a2, const float *__restrict__ w1,
                                                                 const float *__restrict__ w2, float w_offset, float eps, T *__restrict__ out1,
-                                                                T *__restrict__ out2, int W) {
+                                                                T *__restrict__ out2, float *__restrict__ out2_f32, int W) {
     __shared__ float red[16];
     const int64_t n = blockIdx.x;
     float *xr = x + n * W;
@@ -81,18 +81,19 @@ __global__ __launch_bounds__(256) void scaled_add_norms_kernel(float *__restrict
         if (a0.y || a1.y || a2.y) xr[c] = v;
         ss += v * v;
     }
-    if (!out1 && !out2) return;
+    if (!out1 && !out2 && !out2_f32) return;
     ss = block_sum_f32(ss, red);
     const float r = 1.0f / sqrtf(ss / (float)W + eps);
     for (int c = threadIdx.x; c < W; c += 256) {
         const float v = xr[c] * r;
         if (out1) st_f(out1 + n * W + c, w1 ? v * (w_offset + w1[c]) : v);
         if (out2) st_f(out2 + n * W + c, w2 ? v * (w_offset + w2[c]) : v);
+        if (out2_f32) out2_f32[n * W + c] = w2 ? v * (w_offset + w2[c]) : v;
     }
 }
 
 extern "C" int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n_addends, const float *w1, const float *w2, float w_offset, float eps,
-                                   void *out1, void *out2, int dtype, int64_t N, int32_t W, void *stream) {
+                                   void *out1, void *out2, float *out2_f32, int dtype, int64_t N, int32_t W, void *stream) {
     if (N <= 0) return JL_OK;
     if (!x || W <= 0 || n_addends < 0 || n_addends > 3 || (n_addends && !addends)) return jl_fail(JL_E_INVALID, "jl_scaled_add_norms: null pointer, bad width or more than 3 addends");
     jl_addend ad[3] = {{nullptr, 0, 0, nullptr}, {nullptr, 0, 0, nullptr}, {nullptr, 0, 0, nullptr}};
@@ -101,7 +102,7 @@ extern "C" int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n
         if (ad[k].y && ad[k].count <= 0) return jl_fail(JL_E_INVALID, "jl_scaled_add_norms: addend %d has no rows", k);
     }
     JL_DISPATCH(dtype, scaled_add_norms_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x, ad[0], ad[1], ad[2], w1, w2, w_offset, eps, (T *)out1,
-                                                                                                      (T *)out2, W));
+                                                                                                      (T *)out2, out2_f32, W));
     return jl_check_launch("scaled_add_norms_kernel");
 }
 

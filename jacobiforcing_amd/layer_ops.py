@@ -397,11 +397,13 @@ def gated_act(z: torch.Tensor, g_col: int, u_col: int, F_: int, kind: int, limit
 
 
 def scaled_add_norms(x: torch.Tensor, addends: Sequence[Tuple[torch.Tensor, Optional[torch.Tensor]]], w1: Optional[torch.Tensor],
-                     w2: Optional[torch.Tensor], w_offset: float, eps: float, out_dtype: Optional[torch.dtype], two: bool = False):
+                     w2: Optional[torch.Tensor], w_offset: float, eps: float, out_dtype: Optional[torch.dtype], two: bool = False,
+                     second_float: bool = False):
     """x (float [N, W], in place) += sum over ``addends`` (y, scale) of scale * y, y [N, W] or [N, S, W] (summed over S) float or
     bfloat16, scale float [W] or None; then, with ``out_dtype``, the RMS norm of the updated x with float weights stored around
     ``w_offset``: x / rms(x) * (w_offset + w1) — and the same with w2 when ``two`` (both sublayers of a layer read one stream).
-    Returns None, the norm, or the pair of norms."""
+    Returns None, the norm, or the pair of norms; with ``second_float`` (and a 16-bit ``out_dtype``) a third tensor: the second norm
+    unrounded, in float (for a float router beside the experts' 16-bit products)."""
     _dev(x)
     n, W = x.shape
     _need(x.dtype == torch.float32 and x.is_contiguous() and len(addends) <= 3, "scaled_add_norms: x contiguous float32 [N, W], at most 3 addends")
@@ -416,8 +418,11 @@ def scaled_add_norms(x: torch.Tensor, addends: Sequence[Tuple[torch.Tensor, Opti
             _need(w.dtype == torch.float32 and w.numel() == W and w.is_contiguous(), "scaled_add_norms: norm weights are float [W]")
     out1 = torch.empty((n, W), dtype=out_dtype, device=x.device) if out_dtype is not None else None
     out2 = torch.empty((n, W), dtype=out_dtype, device=x.device) if out_dtype is not None and two else None
+    out2f = torch.empty((n, W), dtype=torch.float32, device=x.device) if out2 is not None and second_float and out_dtype != torch.float32 else None
     N.check_layers(N.layers().jl_scaled_add_norms(_ptr(x), arr, len(addends), _ptr(w1), _ptr(w2), float(w_offset), float(eps), _ptr(out1), _ptr(out2),
-                                                 _code(out_dtype or torch.float32), n, W, _stream(x.device)), "jl_scaled_add_norms")
+                                                 _ptr(out2f), _code(out_dtype or torch.float32), n, W, _stream(x.device)), "jl_scaled_add_norms")
+    if two and second_float:
+        return out1, out2, out2f if out2f is not None else out2
     return (out1, out2) if two else out1
 
 

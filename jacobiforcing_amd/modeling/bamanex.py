@@ -263,13 +263,14 @@ class BamanexModel:
         return F.linear(a, w["w_o"], w["b_o"])
 
     # ---- feed-forward: the addends (tensor, channel scale) its result contributes to the residual sum -----------------------------------
-    def _feed_forward(self, li: int, h: torch.Tensor) -> list:
+    def _feed_forward(self, li: int, h: torch.Tensor, h_float: Optional[torch.Tensor] = None) -> list:
+        """``h_float``: the same norm output unrounded (float), when the caller has it: the router reads that."""
         f, w = self.cfg.layers[li]["mlp"], self.w.layers[li]
         if f.get("kind", "dense") == "dense":
             ff = int(f["ff"])
             return [(F.linear(LO.gated_act(F.linear(h, w["w_gu"]), 0, ff, ff, LO.ACT_GELU_TANH), w["w_down"]), w["ls2"])]
         unit = lambda c: (LO.ACT_CLAMPED_SWISH, float(c["limit"]), SWISH_ALPHA, UNIT_SHIFT)
-        out = [(LO.moe_experts(h, F.linear(h.float(), w["router"]), None, int(f["router"]["top"]), 1.0, w["w_gu"], w["w_down"], route="softmax_renorm",
+        out = [(LO.moe_experts(h, F.linear(h_float if h_float is not None else h.float(), w["router"]), None, int(f["router"]["top"]), 1.0, w["w_gu"], w["w_down"], route="softmax_renorm",
                                renorm_eps=ROUTER_RENORM_EPS, gated=unit(f["expert"])), w["ls2"])]
         if f.get("shared") is not None:                 # the token gate multiplies the activation: down() is linear, so the result is the gated output
             fs = int(f["shared"]["ff"])
@@ -291,11 +292,12 @@ class BamanexModel:
         for run, li in enumerate(self.runs):
             L, lw = cfg.layers[li], w.layers[li]
             has_ff = L.get("mlp") is not None
-            hs = LO.scaled_add_norms(x, pending, lw["norm1"], lw["norm2"] if has_ff else None, 1.0, eps, dt, two=has_ff)
-            h1, h2 = hs if has_ff else (hs, None)
+            routed = has_ff and L["mlp"].get("kind", "dense") == "moe"      # a router reads its norm in float, the products the activation dtype
+            hs = LO.scaled_add_norms(x, pending, lw["norm1"], lw["norm2"] if has_ff else None, 1.0, eps, dt, two=has_ff, second_float=routed)
+            h1, h2, h2f = (hs if routed else (*hs, None)) if has_ff else (hs, None, None)
             pending = [(self._attention(run, li, h1, batch, cache), lw["ls1"])]
             if has_ff:
-                pending += self._feed_forward(li, h2)
+                pending += self._feed_forward(li, h2, h2f)
             if trace is not None:
                 LO.scaled_add_norms(x, pending, None, None, 1.0, eps, None)
                 pending = []

@@ -245,6 +245,12 @@ def test_scaled_residual_sum_and_the_two_norms(W):
     newb = x.double() + y1.bfloat16().double()
     assert xb.dtype == torch.float32 and rel_err(xb.cpu(), newb) < 1e-6 and rel_err(ob.float().cpu(), O.centred_norm(newb, w1.double(), 1e-5)) < 6e-3
     assert rel_err(LO.scaled_add_norms(xb, [], w2.cuda(), None, 1.0, 1e-5, torch.float32).cpu(), O.centred_norm(newb, w2.double(), 1e-5)) < 1e-6
+    # the second norm in both forms: rounded for the products, unrounded for a float router
+    p1, p2, p2f = LO.scaled_add_norms(xb, [], w1.cuda(), w2.cuda(), 1.0, 1e-5, torch.bfloat16, two=True, second_float=True)
+    assert p2.dtype == torch.bfloat16 and p2f.dtype == torch.float32 and rel_err(p2f.cpu(), O.centred_norm(newb, w2.double(), 1e-5)) < 1e-6
+    assert torch.equal(p2.cpu(), p2f.cpu().bfloat16()) and rel_err(p1.float().cpu(), O.centred_norm(newb, w1.double(), 1e-5)) < 6e-3
+    q1, q2, q2f = LO.scaled_add_norms(xb, [], w1.cuda(), w2.cuda(), 1.0, 1e-5, torch.float32, two=True, second_float=True)
+    assert q2f is q2 and q2.dtype == torch.float32
     assert LO.scaled_add_norms(xb, [(y3.cuda(), s1.cuda())], None, None, 1.0, 1e-5, None) is None
     assert rel_err(xb.cpu(), newb + y3.double() * s1.double()) < 1e-6
     tiny = torch.full((1, W), 1e-4)                                                            # eps inside the root decides here
