@@ -110,6 +110,11 @@ JL_API int jl_attn_sweep(const jl_attn_args *a, void *stream);
 JL_API int jl_attn_sweep_tile_rows(int dtype, int32_t H, int32_t G, int32_t Gv, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld,
                                    int32_t v_in_k);
 JL_API int64_t jl_attn_sweep_scratch_floats(int32_t n_tiles, int32_t H, int32_t G, int32_t Dv, int32_t splits);
+/* Long portions: with tiles of jl_attn_sweep_wide_tile_rows queries (0: sizes not taken — key widths up to 256, value widths up to 128) and
+ * splits <= 1, jl_attn_sweep runs the form in which a workgroup owns up to 128 (query, head) rows and every wavefront keeps its 32
+ * rows to itself (scores, weights and outputs never leave its registers). */
+JL_API int jl_attn_sweep_wide_tile_rows(int dtype, int32_t H, int32_t G, int32_t Gv, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld,
+                                        int32_t v_in_k);
 
 /* Sublayer-output norm + residual update: x[n] += y[n] / sqrt(mean(y[n]^2) + eps) * g[0] (x float in place, y of y_dtype, g one
  * float); when `out` is given, out[n] = x[n] in `out_dtype` (what the next sublayer's product reads). */

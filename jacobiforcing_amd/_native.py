@@ -264,6 +264,7 @@ _LAYER_SIGNATURES = {
     "jl_attn_sweep": (C.c_int, [C.POINTER(AttnArgs), _vp]),
     "jl_attn_sweep_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32, _i32, _i64, _i64, _i32]),
     "jl_attn_sweep_scratch_floats": (_i64, [_i32, _i32, _i32, _i32, _i32]),
+    "jl_attn_sweep_wide_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32, _i32, _i64, _i64, _i32]),
     "jl_norm_add": (C.c_int, [_vp, _vp, C.c_int, _vp, _f32, _vp, C.c_int, _i64, _i32, _vp]),
     "jl_polynorm": (C.c_int, [_vp, C.c_int, _i64, _i32, _vp, _f32, _vp, _vp]),
     "jl_causal_conv": (C.c_int, [_vp, _vp, C.c_int, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp]),

@@ -19,6 +19,7 @@ from . import _native as N
 ATTN_SPLIT_BELOW_TILES, ATTN_SPLIT_WORKGROUPS = 128, 512     # attention: split a tile's keys while tiles x splits stays below ~2 per CU
 ATTN_MAX_HEADS_ONE_LAUNCH, ATTN_MAX_VALUE_WIDTH = 16, 128   # what the matrix-core attention kernel takes in one workgroup
 SWEEP_SPLIT_BELOW_GROUPS, SWEEP_SPLIT_WORKGROUPS = 512, 2048   # one-sweep attention: its workgroups are small (4 wavefronts, <= 32 rows)
+SWEEP_WIDE_ROWS_PER_REQUEST = 16   # one-sweep attention: from this many tokens per request on average a step takes the 128-row tiles
 RETENTION_CHUNK = 64          # tokens per chunk when a long portion's recurrence is cut into chunks that run side by side
 
 
@@ -274,7 +275,13 @@ def attn_sweep(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ba
     # few tiles with many keys (decoding): share each tile's keys out over workgroups until the chip is full
     groups = tiles.shape[0] * G * -(-(H // G) // 32)
     splits, scratch = 1, None
-    if groups < SWEEP_SPLIT_BELOW_GROUPS:
+    if groups >= SWEEP_SPLIT_BELOW_GROUPS and n >= SWEEP_WIDE_ROWS_PER_REQUEST * batch.B:
+        # long portions: tiles of up to 128 (query, head) rows, every wavefront keeps its rows to itself
+        wide = int(N.layers().jl_attn_sweep_wide_tile_rows(_code(q.dtype), H, G, Gv, D, Dv, k_cache.stride(0), v_cache.stride(0),
+                                                           int(v_cache.data_ptr() == k_cache.data_ptr())))
+        if wide > 0:
+            tq, tiles = wide, batch.tiles(wide)
+    elif groups < SWEEP_SPLIT_BELOW_GROUPS:
         reach = batch.max_pos if window <= 0 else min(batch.max_pos, int(window) + tq)
         splits = max(1, min(-(-reach // 128), SWEEP_SPLIT_WORKGROUPS // groups, 64))
         if splits > 1:

@@ -351,6 +351,39 @@ def test_the_mixer_alone_in_portions_and_single_tokens(H, G, D, Dv, size, dims):
 
 
 @gpu
+@pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 64), (8, 8, 64, 32), (2, 1, 128, 128), (40, 1, 16, 32), (16, 2, 64, 128), (2, 2, 256, 64), (6, 2, 24, 96),
+                                      (3, 1, 40, 128), (8, 2, 128, 128), (5, 1, 64, 32)])
+@pytest.mark.parametrize("size", [0, 21, 100])
+def test_long_portions_on_tiles_of_128_rows(H, G, D, Dv, size, monkeypatch):
+    """bfloat16 steps whose requests bring many tokens run the one-sweep attention on tiles of up to 128 (query, head) rows, every
+    wavefront with rows of its own: two unequal requests side by side, the second continuing from a position inside a page, tiles
+    that end inside a request, windows shorter and longer than a tile, sinks that matter, the head gate."""
+    from jacobiforcing_amd import _native as N
+    from jacobiforcing_amd import layer_ops as LO
+    monkeypatch.setattr(LO, "SWEEP_SPLIT_BELOW_GROUPS", 1)                                      # small steps too
+    assert N.layers().jl_attn_sweep_wide_tile_rows(N.JL_BF16, H, G, G, D, Dv, G * D, G * Dv, 0) == 128 // min(H // G, 32)
+    cfg = one_layer(H, G, D, Dv, size, 8)
+    t = tensors_for(cfg, H + Dv)
+    t["l0.mix.sink"] = t["l0.mix.sink"] + 2.0
+    m = cfg["layers"][0]["mixer"]
+    P = {k: v.double() for k, v in O.layer_tensors(t, 0).items()}
+    ha = torch.randn(170, 64, generator=torch.Generator().manual_seed(1)).bfloat16()
+    hb = torch.randn(107, 64, generator=torch.Generator().manual_seed(2)).bfloat16()
+    want_a, want_b = O.gated_sink_attention(ha.double(), P, m, 1e-5), O.gated_sink_attention(hb.double(), P, m, 1e-5)
+    rig = Rig(cfg, tensors=t, dtype=torch.bfloat16, page=16, pages=32)
+    rig.poison()
+    ta, tb = [9, 3, 20, 11, 5, 0, 1, 2, 4, 6, 30], [7, 8, 10, 12, 13, 14, 15]
+    b0 = rig.LO.RaggedBatch.build([37], [0], [0], [tb], 16, "cuda")                               # the second request's first 37 tokens
+    g0 = rig.model._attention(0, 0, hb[:37].cuda(), b0, rig.cache).float().cpu()
+    b1 = rig.LO.RaggedBatch.build([170, 70], [0, 37], [1, 0], [ta, tb], 16, "cuda")
+    g1 = rig.model._attention(0, 0, torch.cat([ha, hb[37:]]).cuda(), b1, rig.cache).float().cpu()
+    assert rel_err(g1[:170], want_a) < 3e-2 and rel_err(torch.cat([g0, g1[170:]]), want_b) < 3e-2
+    monkeypatch.setenv("JL_ATTN_NO_SWEEP", "1")                                                  # and the two kernels agree to rounding
+    g2 = rig.model._attention(0, 0, torch.cat([ha, hb[37:]]).cuda(), b1, rig.cache).float().cpu()
+    assert rel_err(g1, g2) < 2e-2
+
+
+@gpu
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 1, 64, 64), (8, 2, 32, 96), (6, 2, 24, 40), (3, 3, 20, 12)])
 @pytest.mark.parametrize("size", [0, 300])
 def test_single_tokens_over_a_long_context_take_the_sink_once(H, G, D, Dv, size):
