@@ -17,7 +17,7 @@ extern "C" {
 #endif
 
 #define JL_API __attribute__((visibility("default")))
-#define JL_VERSION 120
+#define JL_VERSION 121
 #define JL_OK 0
 #define JL_E_INVALID (-1)
 #define JL_E_LAUNCH (-3)

@@ -231,6 +231,7 @@ def raise_state_error(code: int, what: str, aux: int = 0):
 
 # ---- libjf_layers.so (include/jf_layers.h): layer kernels of the models whose forward is not stock PyTorch ----------------------------
 JL_F32, JL_BF16 = 0, 1
+JL_VERSION = 121                 # include/jf_layers.h: a library of another version is not called (its signatures may differ)
 JL_OUT_SAME, JL_OUT_F32 = 0, 2
 JL_ACT_GELU_TANH, JL_ACT_CLAMPED_SWISH = 0, 1
 JL_ROUTE_SIGMOID, JL_ROUTE_SOFTMAX_RENORM = 0, 1
@@ -324,6 +325,9 @@ class _LayerLibs:
             except AttributeError as e:
                 raise NativeLibraryError(f"{p} does not export {name}") from e
             fn.restype, fn.argtypes = res, args
+        if int(lib_.jl_version()) != JL_VERSION:
+            raise NativeLibraryError(f"{p} has version {int(lib_.jl_version())}, this package calls version {JL_VERSION}: build it again "
+                                     "(python -c 'import __graft_entry__ as g; g.build()')")
         self._libs[group] = lib_
         return lib_
 
