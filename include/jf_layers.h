@@ -17,7 +17,7 @@ extern "C" {
 #endif
 
 #define JL_API __attribute__((visibility("default")))
-#define JL_VERSION 121
+#define JL_VERSION 122
 #define JL_OK 0
 #define JL_E_INVALID (-1)
 #define JL_E_LAUNCH (-3)
@@ -51,9 +51,13 @@ JL_API int jl_scaled_add_norms(float *x, const jl_addend *addends, int32_t n_add
  * g_col / u_col):   out[n, c] = act(g) * lin(u) * sigmoid(row_gate[n * rg_ld])        (row_gate null: no row gate)
  *   JL_ACT_GELU_TANH:      act(g) = 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), lin(u) = u
  *   JL_ACT_CLAMPED_SWISH:  g' = min(g, limit), u' = clamp(u, -limit, limit); act = g' sigmoid(alpha g'), lin = u' + shift
+ * u_col < 0: the unit has no linear branch (out = act(g), a plain activation).
  * z, row_gate and out [N, F] of `dtype`; the arithmetic is float. */
 #define JL_ACT_GELU_TANH 0
 #define JL_ACT_CLAMPED_SWISH 1
+#define JL_ACT_SILU 2             /* act(g) = g sigmoid(g), lin(u) = u */
+#define JL_ACT_GELU_ERF 3         /* act(g) = 0.5 g (1 + erf(g / sqrt 2)), lin(u) = u */
+#define JL_ACT_NONE (-1)          /* where an activation is optional (jl_short_conv) */
 JL_API int jl_gated_act(const void *z, int dtype, int64_t N, int64_t ld, int32_t g_col, int32_t u_col, int32_t F, int32_t kind, float limit,
                         float alpha, float shift, const void *row_gate, int64_t rg_ld, void *out, void *stream);
 
@@ -116,6 +120,26 @@ JL_API int64_t jl_attn_sweep_scratch_floats(int32_t n_tiles, int32_t H, int32_t 
 JL_API int jl_attn_sweep_wide_tile_rows(int dtype, int32_t H, int32_t G, int32_t Gv, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld,
                                         int32_t v_in_k);
 
+/* Residual update, weighted sum over the streams of all depths, RMS norm — the layer whose result is kept beside the results of all
+ * layers before it, and whose successor reads a learned mixture of them:
+ *   y[n] = x_in[n] + mult * sum_a scale_a * sum_s y_a[n, s]                       (addends as for jl_scaled_add_norms; at most 3)
+ *   depth >= 0:  streams[depth][n] = y[n];  x_out[n] = sum_{j <= depth} mix[j] * streams[j][n]   (mix null: x_out = y)
+ *   depth <  0:  x_out[n] = y[n]              (no addends: nothing is stored, the norm reads x_in)
+ *   out[n] = x_out[n] / sqrt(mean(x_out[n]^2) + eps) * w     in `dtype`, and / or unrounded in out_f32 (either may be null; w null = 1)
+ * streams: float, stream j at streams + j * stream_ld.  x_out may be x_in but must not lie inside streams[0 .. depth]. */
+JL_API int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, int32_t n_addends, float mult, float *streams, int64_t stream_ld,
+                             int32_t depth, const float *mix, float *x_out, const float *w, float eps, void *out, int dtype, float *out_f32,
+                             int64_t N, int32_t W, void *stream);
+
+/* Token shift: out[t] = h[t] + (h[t-1] - h[t]) * mu, element by element, h float [N, W], mu float [W], out [N, W] of `dtype`.  h[t-1] of
+ * a request's first row is tail[slot] (float [slots, W]) when the request has a past (pos0 > 0) and zero otherwise; tail[slot] then
+ * becomes the h of the request's last row of this step.  row_req [N] int32, seq [B, 4] as above. */
+JL_API int jl_token_shift(const float *h, const float *mu, const int32_t *row_req, const int32_t *seq, float *tail, int64_t N, int32_t W,
+                          void *out, int dtype, void *stream);
+
+/* z <- cap * tanh(z / cap) in place over `total` floats (soft cap of the logits). */
+JL_API int jl_softcap(float *z, int64_t total, float cap, void *stream);
+
 /* Sublayer-output norm + residual update: x[n] += y[n] / sqrt(mean(y[n]^2) + eps) * g[0] (x float in place, y of y_dtype, g one
  * float); when `out` is given, out[n] = x[n] in `out_dtype` (what the next sublayer's product reads). */
 JL_API int jl_norm_add(float *x, const void *y, int y_dtype, const float *g, float eps, void *out, int out_dtype, int64_t N, int32_t W,
@@ -136,6 +160,14 @@ JL_API int jl_polynorm(const void *z, int dtype, int64_t N, int32_t F, const flo
 JL_API int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, float *tail,
                           int64_t N, int32_t W, int32_t taps, void *out, void *stream);
 JL_API int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t B, float *tail, int32_t W, int32_t taps, void *stream);
+
+/* Short causal convolution over time of a column range of a product, with an activation and no residual:
+ *   out[t, c] = act(sum_{j < taps} w[c, j] * x[t - taps + 1 + j, col + c])        (zeros before the sequence's start)
+ * x [N, ld] and w [C, taps] of `dtype`, out float [N, C]; act JL_ACT_SILU or JL_ACT_NONE; taps <= 8.  tail float [slots, taps - 1, C] as for
+ * jl_causal_conv (the INPUTS at the positions before the step); it is moved on here as well — for requests with one row in the launch
+ * itself, for the others (max_count > 1) by a second launch enqueued behind it. */
+JL_API int jl_short_conv(const void *x, int dtype, int64_t ld, int32_t col, const void *w, const int32_t *row_req, const int32_t *seq, int32_t B,
+                         int32_t max_count, float *tail, int64_t N, int32_t C, int32_t taps, int32_t act, float *out, void *stream);
 
 /* Per-head query / key stage for attention with M score maps per head: rotation, norm, query temperature, cache append.  proj
  * [N, ld] holds q (H heads x M maps x D at q_col, head by head), k (G x M x D at k_col) and v (G x Dv at v_col).  With rot_dims > 0
@@ -161,16 +193,20 @@ JL_API int jl_diff_combine(const float *a1, const float *a2, int64_t ld, int64_t
  *   cq_out [N, Rq] = rms_norm(query latent) * wq
  *   pool[slot[n]] = [rms_norm(key/value latent) * wkv (R) | rotate(rotary key, pos[n]) (rd)]          (pool rows of R + rd)
  * rotate: of the first rot_dims dimensions, i and i + rot_dims/2 form a pair (u, v) -> (u cos a - v sin a, v cos a + u sin a),
- * a from the cos / sin tables [positions, rot_dims/2] float; the rest pass unchanged. */
+ * a from the cos / sin tables [positions, rot_dims/2] float; the rest pass unchanged (`pairing` JL_ROT_NEIGHBOURS: 2i and 2i + 1 form
+ * the pair instead).  Rq = 0: the model has no query latent (wq, cq_out null; nothing is read at q_col). */
+#define JL_ROT_HALVES 0          /* dimension i pairs with i + rot_dims/2 */
+#define JL_ROT_NEIGHBOURS 1      /* dimension 2i pairs with 2i + 1 (angle i) */
 JL_API int jl_latent_prep(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t Rq, int32_t kv_col, int32_t R,
                           int32_t rd, int32_t rot_dims, const void *wq, const void *wkv, float eps, const int32_t *pos,
                           const float *cos_t, const float *sin_t, int64_t table_len, void *cq_out, void *pool, const int64_t *slot,
-                          void *stream);
+                          int32_t pairing, void *stream);
 /* Queries of latent attention in the pool's coordinates: q_out[n, h] = [qa[h, n, :R] | rotate(q[n, h, D : D + rd], pos[n])] with qa
- * [H, N, R] the unrotated query parts already multiplied by the key up-projection, q [N, H, D + rd]. */
-JL_API int jl_latent_q_pack(const void *qa, const void *q, int dtype, int64_t N, int32_t H, int32_t D, int32_t R, int32_t rd,
+ * [H, N, R] the unrotated query parts already multiplied by the key up-projection, q [N, H, D + rd] with rows q_ld elements apart (a
+ * column range of a wider product). */
+JL_API int jl_latent_q_pack(const void *qa, const void *q, int64_t q_ld, int dtype, int64_t N, int32_t H, int32_t D, int32_t R, int32_t rd,
                             int32_t rot_dims, const int32_t *pos, const float *cos_t, const float *sin_t, int64_t table_len, void *q_out,
-                            void *stream);
+                            int32_t pairing, void *stream);
 /* out[n, h*Dv + d] = ov[h, n, d] * sigmoid(gate[n * gate_ld + h*Dv + d]) (gate null: no gate). */
 JL_API int jl_heads_gate(const void *ov, const void *gate, int64_t gate_ld, int dtype, int64_t N, int32_t H, int32_t Dv, void *out,
                          void *stream);
@@ -198,13 +234,29 @@ JL_API int jl_retention(const void *proj, int dtype, int64_t ld, int32_t q_col, 
 JL_API int jl_retention_join(const int32_t *req, int32_t B, const int32_t *chunk_len, int32_t H, int32_t D, int32_t Dv,
                              const float *decay, float *state, float *scratch, void *stream);
 
+/* Gated delta rule over the ragged batch, state carried in float.  Per head h (key head c = h / (H / G)) and token t:
+ *   q, k = unit vectors (x / sqrt(sum x^2 + unit_eps)) of the head's D query / key values, q also times q_scale;
+ *   beta = sigmoid(b_h(t));   g = exp(-exp(A_log[h]) * softplus(a_h(t) + dt_bias[h]));
+ *   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q            (S [D, Dv]; the read-out sees the token's own write)
+ *   out_h(t) = o / sqrt(mean(o^2) + eps) * norm_w * silu(gate_h(t))             (norm_w float [Dv], shared by the heads)
+ * qkv float [N, qkv_ld] holds q, k (G*D columns each) and v (H*Dv) after their convolution and activation; proj [N, ld] of `dtype` holds
+ * a, b (H columns each) and the gate (H*Dv).  state [slots, H, D, Dv] float: a request with pos0 == 0 starts from zero (its slot's old
+ * content is ignored); the final state is written back.  out [N, H*Dv] of `dtype`.  D <= 256, Dv <= 1024. */
+JL_API int jl_delta_rule(const void *qkv, int qkv_dtype, int64_t qkv_ld, int32_t q_col, int32_t k_col, int32_t v_col, const void *proj, int dtype,
+                         int64_t ld, int32_t a_col, int32_t b_col, int32_t g_col, const float *A_log, const float *dt_bias, const float *norm_w,
+                         const int32_t *seq, int32_t B, int32_t H, int32_t G, int32_t D, int32_t Dv, float unit_eps, float q_scale, float eps,
+                         float *state, void *out, void *stream);
+
 /* Router of a mixture of experts over float logits [N, E]; ids [N, top] int32, weights [N, top] float.
  *   JL_ROUTE_SIGMOID:        s = sigmoid(logits); the `top` experts with the largest s + correction are chosen (ties: lowest
  *                            index); weights = s * scale (not renormalised).
  *   JL_ROUTE_SOFTMAX_RENORM: s = softmax(logits) over all experts; the `top` largest are chosen (ties: lowest index); weights =
- *                            s / (sum of the chosen s + renorm_eps) * scale.  `correction` is not read. */
+ *                            s / (sum of the chosen s + renorm_eps) * scale.  `correction` is not read.
+ *   JL_ROUTE_TOP_SOFTMAX:    the `top` largest logits are chosen (ties: lowest index); weights = softmax over the chosen logits
+ *                            only, times scale.  `correction` is not read. */
 #define JL_ROUTE_SIGMOID 0
 #define JL_ROUTE_SOFTMAX_RENORM 1
+#define JL_ROUTE_TOP_SOFTMAX 2
 JL_API int jl_moe_route(const float *logits, const float *correction, int64_t N, int32_t E, int32_t top, float scale, int32_t *ids,
                         float *weights, int32_t kind, float renorm_eps, void *stream);
 

@@ -18,10 +18,10 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibilit
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
 # The layer kernels come in two libraries, so that a model compiles (at the first call of a fresh checkout) only what it launches:
-# "layers" = norms, convolution, attention and its input / output stages; "layers_seq" = the recurrent mixer and the routed experts.
+# "layers" = norms, convolution, attention and its input / output stages; "layers_seq" = the recurrent mixers and the routed experts.
 LAYER_GROUPS = {
     "layers": ["jl_error", "jl_norm", "jl_conv", "jl_headnorm", "jl_latent", "jl_attn_sweep", "jl_attn"],
-    "layers_seq": ["jl_error", "jl_retention", "jl_moe"],
+    "layers_seq": ["jl_error", "jl_retention", "jl_delta", "jl_moe"],
 }
 LAYERS_HEADERS = [CSRC / "layers" / "jl_common.h", ROOT / "include" / "jf_layers.h"]
 

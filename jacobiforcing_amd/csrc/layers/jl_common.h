@@ -55,8 +55,12 @@ __device__ __forceinline__ float block_sum_f32(float v, float *red) {
 __device__ __forceinline__ float gelu_tanh_f(float z) {
     return z / (1.0f + expf(-1.5957691216057308f * (z + 0.044715f * z * z * z)));
 }
+__device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float gated_unit_f(float g, float u, int kind, float limit, float alpha, float shift) {
     if (kind == JL_ACT_GELU_TANH) return gelu_tanh_f(g) * u;
+    if (kind == JL_ACT_SILU) return silu_f(g) * u;
+    if (kind == JL_ACT_GELU_ERF) return gelu_erf_f(g) * u;
     g = fminf(g, limit);                                            // clamped swish: the gate capped from above, the linear branch from both sides
     u = fminf(fmaxf(u, -limit), limit);
     return g / (1.0f + expf(-alpha * g)) * (u + shift);

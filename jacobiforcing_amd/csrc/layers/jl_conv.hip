@@ -138,3 +138,96 @@ extern "C" int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t 
     causal_conv_carry_kernel<<<dim3((unsigned)((W + 255) / 256), (unsigned)B), 256, 0, (hipStream_t)stream>>>(x, seq, tail, W, taps);
     return jl_check_launch("causal_conv_carry_kernel");
 }
+
+// ---- short causal convolution of a column range of a projection, with an activation, no residual ---------------------------------------------
+//   out[t, c] = act(sum_{j < taps} w[c, j] * x[t - taps + 1 + j, col + c])        (zeros before the sequence's start; float out)
+// A workgroup walks CONV_ROWS consecutive rows, a thread owns a channel and keeps the last taps - 1 inputs in registers.  The tail
+// (float [slots, taps - 1, C]) is read for the inputs before the step and moved on here by requests with ONE row; requests with more rows
+// leave that to short_conv_carry_kernel, enqueued after every row has read.
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void short_conv_kernel(const T *__restrict__ x, int64_t ld, int col, const T *__restrict__ w, const int32_t *__restrict__ row_req,
+                                                          const int32_t *__restrict__ seq, float *tail, int64_t N, int C, int act, float *__restrict__ out) {
+    constexpr int KEEP = TAPS - 1;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    float wv[TAPS], win[KEEP > 0 ? KEEP : 1];
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) wv[j] = ld_f(w + (int64_t)c * TAPS + j);
+    int prev_req = -1;
+    const int64_t n0 = (int64_t)blockIdx.x * CONV_ROWS;
+    for (int r = 0; r < CONV_ROWS && n0 + r < N; ++r) {
+        const int64_t n = n0 + r;
+        const int req = row_req[n];
+        const int32_t *rec = seq + 4 * (int64_t)req;
+        const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3];
+        const int t = (int)(n - row0);
+        if (req != prev_req) {
+#pragma unroll
+            for (int s2 = 0; s2 < KEEP; ++s2) {
+                const int u = t - KEEP + s2;
+                float v = 0.f;
+                if (u >= 0) v = ld_f(x + (int64_t)(row0 + u) * ld + col + c);
+                else if (pos0 + u >= 0) v = tail[((int64_t)slot * KEEP + (KEEP + u)) * C + c];
+                win[s2] = v;
+            }
+            prev_req = req;
+        }
+        const float cur = ld_f(x + n * ld + col + c);
+        float a = wv[KEEP] * cur;
+#pragma unroll
+        for (int s2 = 0; s2 < KEEP; ++s2) a += wv[s2] * win[s2];
+        out[n * C + c] = act == JL_ACT_SILU ? silu_f(a) : a;
+#pragma unroll
+        for (int s2 = 0; s2 + 1 < KEEP; ++s2) win[s2] = win[s2 + 1];
+        if (KEEP > 0) win[KEEP - 1] = cur;
+        if (count == 1 && KEEP > 0) {
+#pragma unroll
+            for (int s2 = 0; s2 < KEEP; ++s2) tail[((int64_t)slot * KEEP + s2) * C + c] = win[s2];
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_carry_kernel(const T *__restrict__ x, int64_t ld, int col, const int32_t *__restrict__ seq,
+                                                                float *__restrict__ tail, int C, int taps) {
+    const int32_t *rec = seq + 4 * (int64_t)blockIdx.y;
+    const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3], keep = taps - 1;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C || count <= 1) return;
+    float v[JL_CONV_MAX_TAPS];
+#pragma unroll
+    for (int s = 0; s < JL_CONV_MAX_TAPS - 1; ++s) {
+        v[s] = 0.f;
+        if (s < keep) {
+            const int u = count - keep + s;
+            if (u >= 0) v[s] = ld_f(x + (int64_t)(row0 + u) * ld + col + c);
+            else if (pos0 + u >= 0) v[s] = tail[((int64_t)slot * keep + (keep + u)) * C + c];
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < JL_CONV_MAX_TAPS - 1; ++s)
+        if (s < keep) tail[((int64_t)slot * keep + s) * C + c] = v[s];
+}
+
+template <typename T, int TAPS>
+static void short_conv_launch(const void *x, int64_t ld, int col, const void *w, const int32_t *row_req, const int32_t *seq, float *tail, int64_t N, int C,
+                              int act, float *out, hipStream_t st) {
+    const dim3 grid((unsigned)((N + CONV_ROWS - 1) / CONV_ROWS), (unsigned)((C + 255) / 256));
+    short_conv_kernel<T, TAPS><<<grid, 256, 0, st>>>((const T *)x, ld, col, (const T *)w, row_req, seq, tail, N, C, act, out);
+}
+
+extern "C" int jl_short_conv(const void *x, int dtype, int64_t ld, int32_t col, const void *w, const int32_t *row_req, const int32_t *seq, int32_t B,
+                             int32_t max_count, float *tail, int64_t N, int32_t C, int32_t taps, int32_t act, float *out, void *stream) {
+    if (N <= 0) return JL_OK;
+    if (!x || !w || !row_req || !seq || !out || C <= 0 || col < 0 || col + (int64_t)C > ld || taps < 1 || taps > 8 || (taps > 1 && !tail))
+        return jl_fail(JL_E_INVALID, "jl_short_conv: null pointer, columns outside the row, or taps outside 1..8");
+    if (act != JL_ACT_SILU && act != JL_ACT_NONE) return jl_fail(JL_E_INVALID, "jl_short_conv: unknown activation %d", act);
+    hipStream_t st = (hipStream_t)stream;
+#define CONV_CASE(TP) case TP: JL_DISPATCH(dtype, (short_conv_launch<T, TP>(x, ld, col, w, row_req, seq, tail, N, C, act, out, st))); break
+    switch (taps) { CONV_CASE(1); CONV_CASE(2); CONV_CASE(3); CONV_CASE(4); CONV_CASE(5); CONV_CASE(6); CONV_CASE(7); CONV_CASE(8); }
+#undef CONV_CASE
+    int rc = jl_check_launch("short_conv_kernel");
+    if (rc != JL_OK || taps == 1 || max_count <= 1) return rc;
+    JL_DISPATCH(dtype, short_conv_carry_kernel<T><<<dim3((unsigned)((C + 255) / 256), (unsigned)B), 256, 0, st>>>((const T *)x, ld, col, seq, tail, C, taps));
+    return jl_check_launch("short_conv_carry_kernel");
+}

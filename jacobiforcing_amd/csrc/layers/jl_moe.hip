@@ -1,4 +1,5 @@
-// jl_moe.hip — routed experts: the router's choice (sigmoid scores with a correction, or a softmax renormalised over the chosen), the
+// jl_moe.hip — routed experts: the router's choice (sigmoid scores with a correction, a softmax renormalised over the chosen, or a
+// softmax over the chosen logits alone), the
 // rows grouped by expert, and the grouped products: up with relu^2 or plain (a gated unit's activation is its own launch), down with
 // the routing weights.
 #include "jl_common.h"
@@ -11,6 +12,26 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
     const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (n >= N) return;
     const float *z = logits + n * E;
+    if (kind == JL_ROUTE_TOP_SOFTMAX) {
+        // the largest `top` logits (ties: lowest index), found in descending order; weights = softmax over the chosen logits only
+        float zmax = 0.f, den = 0.f;
+        for (int s = 0; s < top; ++s) {
+            int best = -1;
+            float bz = 0.f;
+            for (int e = 0; e < E; ++e) {
+                bool taken = false;
+                for (int p = 0; p < s; ++p) taken |= ids[n * top + p] == e;
+                if (!taken && (best < 0 || z[e] > bz)) { best = e; bz = z[e]; }
+            }
+            if (s == 0) zmax = bz;
+            const float w = expf(bz - zmax);
+            ids[n * top + s] = best;
+            weights[n * top + s] = w;
+            den += w;
+        }
+        for (int s = 0; s < top; ++s) weights[n * top + s] = weights[n * top + s] / den * scale;
+        return;
+    }
     if (kind == JL_ROUTE_SOFTMAX_RENORM) {
         // scores = softmax over ALL experts; the largest `top` (ties: lowest index); weights = score / (sum of the chosen + renorm_eps)
         float zmax = -INFINITY, den = 0.f, chosen = 0.f;
@@ -52,7 +73,7 @@ extern "C" int jl_moe_route(const float *logits, const float *correction, int64_
                             float *weights, int32_t kind, float renorm_eps, void *stream) {
     if (N <= 0) return JL_OK;
     if (!logits || !ids || !weights || E <= 0 || top <= 0 || top > E) return jl_fail(JL_E_INVALID, "jl_moe_route: null pointer or top > experts");
-    if (kind != JL_ROUTE_SIGMOID && kind != JL_ROUTE_SOFTMAX_RENORM) return jl_fail(JL_E_INVALID, "jl_moe_route: unknown kind %d", kind);
+    if (kind < JL_ROUTE_SIGMOID || kind > JL_ROUTE_TOP_SOFTMAX) return jl_fail(JL_E_INVALID, "jl_moe_route: unknown kind %d", kind);
     moe_route_kernel<<<dim3((unsigned)((N + 255) / 256)), 256, 0, (hipStream_t)stream>>>(logits, correction, N, E, top, scale, ids, weights, kind,
                                                                                          renorm_eps);
     return jl_check_launch("moe_route_kernel");
@@ -324,7 +345,7 @@ extern "C" int jl_moe_gemm_gated(const void *X, const void *Wt, int dtype, int32
                                  float limit, float alpha, float shift, void *out, void *stream) {
     if (max_tiles <= 0) return JL_OK;
     if (!X || !Wt || !perm || !offsets || !tile_expert || !tile_row0 || !out) return jl_fail(JL_E_INVALID, "jl_moe_gemm_gated: null pointer");
-    if (K <= 0 || ff <= 0 || top <= 0 || (kind != JL_ACT_GELU_TANH && kind != JL_ACT_CLAMPED_SWISH))
+    if (K <= 0 || ff <= 0 || top <= 0 || kind < JL_ACT_GELU_TANH || kind > JL_ACT_GELU_ERF)
         return jl_fail(JL_E_INVALID, "jl_moe_gemm_gated: bad sizes or kind");
     const MoeAct act = {kind, limit, alpha, shift};
     return moe_gemm_launch(X, Wt, dtype, JL_MOE_UP_PLAIN, K, ff, top, perm, offsets, tile_expert, tile_row0, max_tiles, nullptr, out, &act, stream);

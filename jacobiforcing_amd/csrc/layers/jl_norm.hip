@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T *__restrict__ z,
     if (e >= total) return;
     const int64_t n = e / F;
     const int c = (int)(e - n * F);
-    float v = gated_unit_f(ld_f(z + n * ld + g_col + c), ld_f(z + n * ld + u_col + c), kind, limit, alpha, shift);
+    float v = gated_unit_f(ld_f(z + n * ld + g_col + c), u_col < 0 ? 1.0f : ld_f(z + n * ld + u_col + c), kind, limit, alpha, shift);
     if (row_gate) v *= 1.0f / (1.0f + expf(-ld_f(row_gate + n * rg_ld)));
     st_f(out + e, v);
 }
@@ -150,7 +150,10 @@ __global__ __launch_bounds__(256) void gated_act_vec_kernel(const T *__restrict_
     const int c = (int)(e - n * per_row) * VEC;
     float g[VEC], u[VEC];
     ld16(z + n * ld + g_col + c, g);
-    ld16(z + n * ld + u_col + c, u);
+    if (u_col >= 0) ld16(z + n * ld + u_col + c, u);
+    else
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) u[i] = 1.0f;
     const float rg = row_gate ? 1.0f / (1.0f + expf(-ld_f(row_gate + n * rg_ld))) : 1.0f;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) g[i] = gated_unit_f(g[i], u[i], kind, limit, alpha, shift) * rg;
@@ -160,11 +163,12 @@ __global__ __launch_bounds__(256) void gated_act_vec_kernel(const T *__restrict_
 extern "C" int jl_gated_act(const void *z, int dtype, int64_t N, int64_t ld, int32_t g_col, int32_t u_col, int32_t F, int32_t kind, float limit, float alpha,
                             float shift, const void *row_gate, int64_t rg_ld, void *out, void *stream) {
     if (N <= 0) return JL_OK;
-    if (!z || !out || F <= 0 || g_col < 0 || u_col < 0 || g_col + (int64_t)F > ld || u_col + (int64_t)F > ld)
+    if (!z || !out || F <= 0 || g_col < 0 || g_col + (int64_t)F > ld || u_col + (int64_t)F > ld)
         return jl_fail(JL_E_INVALID, "jl_gated_act: null pointer, or the columns do not fit the row stride");
-    if (kind != JL_ACT_GELU_TANH && kind != JL_ACT_CLAMPED_SWISH) return jl_fail(JL_E_INVALID, "jl_gated_act: unknown kind %d", kind);
+    if (kind < JL_ACT_GELU_TANH || kind > JL_ACT_GELU_ERF) return jl_fail(JL_E_INVALID, "jl_gated_act: unknown kind %d", kind);
+    if (u_col < 0) u_col = -1;
     const int vec = dtype == JL_BF16 ? 8 : 4;
-    if (F % vec == 0 && g_col % vec == 0 && u_col % vec == 0 && ld % vec == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    if (F % vec == 0 && g_col % vec == 0 && (u_col < 0 || u_col % vec == 0) && ld % vec == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
         const int64_t vecs = N * (F / vec);
         JL_DISPATCH(dtype, gated_act_vec_kernel<T><<<dim3((unsigned)((vecs + 255) / 256)), 256, 0, (hipStream_t)stream>>>(
                                (const T *)z, ld, g_col, u_col, F, kind, limit, alpha, shift, (const T *)row_gate, rg_ld, (T *)out, vecs));
@@ -238,4 +242,113 @@ extern "C" int jl_polynorm(const void *z, int dtype, int64_t N, int32_t F, const
     if (!z || !coef || !out || F <= 0) return jl_fail(JL_E_INVALID, "jl_polynorm: null pointer or bad width");
     JL_DISPATCH(dtype, polynorm_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>((const T *)z, F, coef, eps, (T *)out));
     return jl_check_launch("polynorm_kernel");
+}
+
+// ---- residual update + weighted sum over the streams of all depths + RMS norm: one workgroup per row ------------------------------------
+// pass 1: y = x_in + mult * (sum of the addends) is stored as stream `depth`; v = sum_j mix[j] * stream_j (j <= depth; the last one from
+// registers) is stored as x_out, with its sum of squares; pass 2: the norm of what pass 1 wrote, in `dtype` and / or unrounded.
+template <typename T>
+__global__ __launch_bounds__(256) void depth_mix_norm_kernel(const float *__restrict__ x_in, jl_addend a0, jl_addend a1, jl_addend a2, float mult,
+                                                              float *__restrict__ streams, int64_t stream_ld, int depth, const float *__restrict__ mix,
+                                                              float *__restrict__ x_out, const float *__restrict__ w, float eps, T *__restrict__ out,
+                                                              float *__restrict__ out_f32, int W) {
+    __shared__ float red[16];
+    const int64_t n = blockIdx.x;
+    const jl_addend ad[3] = {a0, a1, a2};
+    const bool update = a0.y || a1.y || a2.y || depth >= 0;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            if (!ad[k].y) continue;
+            float u = 0.f;
+            for (int s = 0; s < ad[k].count; ++s) u += ld_any(ad[k].y, ad[k].dtype, (n * ad[k].count + s) * (int64_t)W + c);
+            t += ad[k].scale ? u * ad[k].scale[c] : u;
+        }
+        float v = x_in[n * W + c] + mult * t;
+        if (depth >= 0) {
+            streams[depth * stream_ld + n * W + c] = v;
+            if (mix) {
+                v *= mix[depth];
+                for (int j = 0; j < depth; ++j) v += mix[j] * streams[j * stream_ld + n * W + c];
+            }
+        }
+        if (update) x_out[n * W + c] = v;
+        ss += v * v;
+    }
+    if (!out && !out_f32) return;
+    ss = block_sum_f32(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)W + eps);
+    const float *xr = update ? x_out + n * W : x_in + n * W;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float v = xr[c] * r * (w ? w[c] : 1.0f);
+        if (out) st_f(out + n * W + c, v);
+        if (out_f32) out_f32[n * W + c] = v;
+    }
+}
+
+extern "C" int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, int32_t n_addends, float mult, float *streams, int64_t stream_ld,
+                                 int32_t depth, const float *mix, float *x_out, const float *w, float eps, void *out, int dtype, float *out_f32,
+                                 int64_t N, int32_t W, void *stream) {
+    if (N <= 0) return JL_OK;
+    if (!x_in || W <= 0 || n_addends < 0 || n_addends > 3 || (n_addends && !addends))
+        return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: null pointer, bad width or more than 3 addends");
+    if ((depth >= 0 || n_addends) && !x_out) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: an updated stream needs x_out");
+    if (depth >= 0 && (!streams || stream_ld < N * (int64_t)W)) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: streams of at least N * W floats each");
+    if (depth >= 0 && x_out >= streams && x_out < streams + (int64_t)(depth + 1) * stream_ld)
+        return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: x_out lies inside the streams it is mixed from");
+    jl_addend ad[3] = {{nullptr, 0, 0, nullptr}, {nullptr, 0, 0, nullptr}, {nullptr, 0, 0, nullptr}};
+    for (int k = 0; k < n_addends; ++k) {
+        ad[k] = addends[k];
+        if (ad[k].y && ad[k].count <= 0) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: addend %d has no rows", k);
+    }
+    JL_DISPATCH(dtype, depth_mix_norm_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x_in, ad[0], ad[1], ad[2], mult, streams, stream_ld, depth,
+                                                                                                    mix, x_out, w, eps, (T *)out, out_f32, W));
+    return jl_check_launch("depth_mix_norm_kernel");
+}
+
+// ---- token shift: out = h + (h of the previous token - h) * mu, the previous token of a request's first row coming from its slot ------------
+// One workgroup per row.  The thread that owns channel c of a request's FIRST row is the only one that touches tail[slot, c] in the
+// launch: it reads the old value (when the request has a past) and then stores the h of the request's last row of this step.
+template <typename T>
+__global__ __launch_bounds__(256) void token_shift_kernel(const float *__restrict__ h, const float *__restrict__ mu, const int32_t *__restrict__ row_req,
+                                                           const int32_t *__restrict__ seq, float *tail, int W, T *__restrict__ out) {
+    const int64_t n = blockIdx.x;
+    const int32_t *rec = seq + 4 * (int64_t)row_req[n];
+    const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3];
+    const bool first = n == row0;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        const float cur = h[n * W + c];
+        float prev;
+        if (first) {
+            float *tl = tail + (int64_t)slot * W + c;
+            prev = pos0 > 0 ? *tl : 0.f;
+            *tl = h[(int64_t)(row0 + count - 1) * W + c];
+        } else {
+            prev = h[(n - 1) * W + c];
+        }
+        st_f(out + n * W + c, cur + (prev - cur) * mu[c]);
+    }
+}
+
+extern "C" int jl_token_shift(const float *h, const float *mu, const int32_t *row_req, const int32_t *seq, float *tail, int64_t N, int32_t W,
+                              void *out, int dtype, void *stream) {
+    if (N <= 0) return JL_OK;
+    if (!h || !mu || !row_req || !seq || !tail || !out || W <= 0) return jl_fail(JL_E_INVALID, "jl_token_shift: null pointer or bad width");
+    JL_DISPATCH(dtype, token_shift_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(h, mu, row_req, seq, tail, W, (T *)out));
+    return jl_check_launch("token_shift_kernel");
+}
+
+// ---- soft cap of the logits, in place: z <- cap * tanh(z / cap) ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void softcap_kernel(float *__restrict__ z, int64_t total, float cap) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e < total) z[e] = cap * tanhf(z[e] / cap);
+}
+
+extern "C" int jl_softcap(float *z, int64_t total, float cap, void *stream) {
+    if (total <= 0) return JL_OK;
+    if (!z || !(cap > 0.f)) return jl_fail(JL_E_INVALID, "jl_softcap: null pointer or a cap that is not positive");
+    softcap_kernel<<<dim3((unsigned)((total + 255) / 256)), 256, 0, (hipStream_t)stream>>>(z, total, cap);
+    return jl_check_launch("softcap_kernel");
 }

@@ -6,8 +6,8 @@ A *layer run* is one execution of a layer in a forward: a model that repeats a s
 run — and therefore one cache or state of its own — per repetition."""
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import List, Optional
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
 
 import torch
 
@@ -17,12 +17,14 @@ class RunSpec:
     """Memory one layer run needs.  kind "kv": ``k_width`` / ``v_width`` elements per cached token (all key/value heads side by
     side; ``v_width`` 0: the values are read out of the key rows, there is no second pool).  kind "state": a float tensor of
     ``state_shape`` per slot.  kind None: nothing.  Beside either, ``tail_shape`` (when not empty) is a small float tensor per slot
-    for what a layer carries from step to step whatever its mixer is (the last inputs of a short convolution)."""
+    for what a layer carries from step to step whatever its mixer is (the last inputs of a short convolution); a layer that carries
+    several such things of different shapes names them in ``tails`` (name -> shape per slot)."""
     kind: Optional[str]
     k_width: int = 0
     v_width: int = 0
     state_shape: tuple = ()
     tail_shape: tuple = ()
+    tails: Dict[str, tuple] = field(default_factory=dict)
 
 
 class PagedStateCache:
@@ -34,6 +36,7 @@ class PagedStateCache:
         self.v: List[Optional[torch.Tensor]] = []
         self.state: List[Optional[torch.Tensor]] = []
         self.tail: List[Optional[torch.Tensor]] = []
+        self.tails: List[Dict[str, torch.Tensor]] = []
         for s in specs:
             kv = s.kind == "kv"
             self.k.append(torch.zeros((tokens, s.k_width), dtype=dtype, device=device) if kv else None)
@@ -41,6 +44,9 @@ class PagedStateCache:
             self.tail.append(torch.zeros((self.num_slots, *s.tail_shape), dtype=torch.float32, device=device)
                              if s.tail_shape and all(int(d) > 0 for d in s.tail_shape) else None)
             self.state.append(torch.zeros((self.num_slots, *s.state_shape), dtype=torch.float32, device=device) if s.kind == "state" else None)
+            self.tails.append({k: torch.zeros((self.num_slots, *shape), dtype=torch.float32, device=device)
+                               for k, shape in s.tails.items() if shape and all(int(d) > 0 for d in shape)})
 
     def bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for ts in (self.k, self.v, self.state, self.tail) for t in ts if t is not None)
+        return (sum(t.numel() * t.element_size() for ts in (self.k, self.v, self.state, self.tail) for t in ts if t is not None) +
+                sum(t.numel() * t.element_size() for d in self.tails for t in d.values()))

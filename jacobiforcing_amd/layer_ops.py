@@ -129,11 +129,15 @@ class RaggedBatch:
         return t
 
 
-def embed_scale(embed: torch.Tensor, ids: torch.Tensor, scale: float, want_copy: bool) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+def embed_scale(embed: torch.Tensor, ids: torch.Tensor, scale: float, want_copy: bool,
+                out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Rows ``ids`` of ``embed`` times ``scale`` as float [N, W] (written into ``out`` when given), and a second copy with ``want_copy``."""
     _dev(embed)
     _need(embed.dim() == 2 and embed.is_contiguous() and ids.dtype == torch.int64 and ids.is_contiguous(), "embed_scale: embed [V, W], ids int64 [N]")
     n, W = ids.numel(), embed.shape[1]
-    x = torch.empty((n, W), dtype=torch.float32, device=embed.device)
+    if out is not None:
+        _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (n, W), "embed_scale: out float [N, W]")
+    x = out if out is not None else torch.empty((n, W), dtype=torch.float32, device=embed.device)
     x0 = torch.empty_like(x) if want_copy else None
     N.check_layers(N.layers().jl_embed_scale(_ptr(embed), _code(embed.dtype), _ptr(ids), n, W, float(scale), _ptr(x), _ptr(x0),
                                             _stream(embed.device)), "jl_embed_scale")
@@ -331,6 +335,9 @@ def retention(proj: torch.Tensor, cols: Tuple[int, int, int, int], batch: Ragged
     return out
 
 
+_ROUTES = {"sigmoid": N.JL_ROUTE_SIGMOID, "softmax_renorm": N.JL_ROUTE_SOFTMAX_RENORM, "top_softmax": N.JL_ROUTE_TOP_SOFTMAX}
+
+
 def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, scale: float,
                 w_up: torch.Tensor, w_down: torch.Tensor, route: str = "sigmoid", renorm_eps: float = 0.0,
                 gated: Optional[Tuple[int, float, float, float]] = None) -> torch.Tensor:
@@ -338,7 +345,8 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
     float [N, top, W] (their sum over the middle axis is the layer's output).
 
     ``route`` "sigmoid": sigmoid scores, choice by score + correction, weights = score * scale; "softmax_renorm": softmax over all
-    experts, the largest chosen, weights = score / (sum of the chosen + renorm_eps) * scale.
+    experts, the largest chosen, weights = score / (sum of the chosen + renorm_eps) * scale; "top_softmax": the largest logits chosen,
+    weights = softmax over the chosen logits only, times scale.
     ``gated`` None: experts down(relu(up h)^2) with w_up [E, ff, W].  ``gated`` = (kind, limit, alpha, shift) of ``gated_act``: w_up
     [E, 2*ff, W] stacks every expert's gate rows on its linear rows, and the up product applies the unit in its epilogue."""
     _dev(h)
@@ -350,14 +358,14 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
           "moe_experts: h [N, W], logits float [N, E]")
     _need(tuple(w_up.shape) == (E, up_rows, W) and tuple(w_down.shape) == (E, W, ff) and w_up.dtype == dt and w_down.dtype == dt and
           w_up.is_contiguous() and w_down.is_contiguous(), "moe_experts: expert weights [E, ff (2*ff when gated), W] / [E, W, ff] in the activation dtype")
-    _need(route in ("sigmoid", "softmax_renorm") and 1 <= top <= E, "moe_experts: route is 'sigmoid' or 'softmax_renorm', 1 <= top <= experts")
+    _need(route in _ROUTES and 1 <= top <= E, "moe_experts: route is 'sigmoid', 'softmax_renorm' or 'top_softmax', 1 <= top <= experts")
     if correction is not None:
         _need(correction.dtype == torch.float32 and correction.numel() == E, "moe_experts: correction float [E]")
     L, st = N.layers(), _stream(dev)
     ids = torch.empty((n, top), dtype=torch.int32, device=dev)
     wts = torch.empty((n, top), dtype=torch.float32, device=dev)
     N.check_layers(L.jl_moe_route(_ptr(router_logits), _ptr(correction), n, E, top, float(scale), _ptr(ids), _ptr(wts),
-                                  N.JL_ROUTE_SIGMOID if route == "sigmoid" else N.JL_ROUTE_SOFTMAX_RENORM, float(renorm_eps), st), "jl_moe_route")
+                                  _ROUTES[route], float(renorm_eps), st), "jl_moe_route")
     tm = int(L.jl_moe_tile_rows())
     rows = n * top
     max_tiles = rows // tm + E
@@ -382,16 +390,18 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
     return y
 
 
-ACT_GELU_TANH, ACT_CLAMPED_SWISH = N.JL_ACT_GELU_TANH, N.JL_ACT_CLAMPED_SWISH
+ACT_GELU_TANH, ACT_CLAMPED_SWISH, ACT_SILU, ACT_GELU_ERF, ACT_NONE = N.JL_ACT_GELU_TANH, N.JL_ACT_CLAMPED_SWISH, N.JL_ACT_SILU, N.JL_ACT_GELU_ERF, N.JL_ACT_NONE
 
 
 def gated_act(z: torch.Tensor, g_col: int, u_col: int, F_: int, kind: int, limit: float = 0.0, alpha: float = 1.0, shift: float = 0.0,
               row_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Gated activation of a feed-forward whose gate and linear branch are F_ columns each of one product z [N, ld], at g_col /
     u_col.  ACT_GELU_TANH: gelu_tanh(g) * u.  ACT_CLAMPED_SWISH: g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(alpha g') (u' +
-    shift).  ``row_gate`` [N] or [N, 1] view (row stride free): the row is further multiplied by sigmoid(row_gate).  Returns [N, F_]."""
+    shift).  ACT_SILU: g sigmoid(g) * u.  ACT_GELU_ERF: 0.5 g (1 + erf(g / sqrt 2)) * u.  ``u_col`` < 0: no linear branch (a plain
+    activation of the F_ columns at g_col).  ``row_gate`` [N] or [N, 1] view (row stride free): the row is further multiplied by sigmoid(row_gate).  Returns [N, F_]."""
     _dev(z)
-    _need(z.dim() == 2 and z.stride(1) == 1 and g_col + F_ <= z.shape[1] and u_col + F_ <= z.shape[1], "gated_act: z [N, ld] with both column ranges inside")
+    u_col = -1 if u_col < 0 else u_col
+    _need(z.dim() == 2 and z.stride(1) == 1 and 0 <= g_col and g_col + F_ <= z.shape[1] and u_col + F_ <= z.shape[1], "gated_act: z [N, ld] with both column ranges inside")
     n = z.shape[0]
     rg_ld = 0
     if row_gate is not None:
@@ -524,33 +534,39 @@ def _angle_tables(rot_dims: int, cos, sin, batch: RaggedBatch, what: str) -> int
     return cos.shape[0]
 
 
-def latent_prep(proj: torch.Tensor, q_col: int, Rq: int, kv_col: int, R: int, rd: int, rot_dims: int, wq: torch.Tensor, wkv: torch.Tensor,
-                eps: float, batch: RaggedBatch, cos, sin, pool: torch.Tensor) -> torch.Tensor:
-    """Normalised query latent [N, Rq]; the pool row of every token becomes [normalised key/value latent | rotated shared key]."""
+ROT_HALVES, ROT_NEIGHBOURS = N.JL_ROT_HALVES, N.JL_ROT_NEIGHBOURS      # which dimensions a rotation pairs: i with i + dims/2, or 2i with 2i + 1
+
+
+def latent_prep(proj: torch.Tensor, q_col: int, Rq: int, kv_col: int, R: int, rd: int, rot_dims: int, wq: Optional[torch.Tensor], wkv: torch.Tensor,
+                eps: float, batch: RaggedBatch, cos, sin, pool: torch.Tensor, pairing: int = N.JL_ROT_HALVES) -> Optional[torch.Tensor]:
+    """Normalised query latent [N, Rq] (None with Rq = 0: a model without one); the pool row of every token becomes [normalised key/value
+    latent | rotated shared key]."""
     _dev(proj)
     n, ld = proj.shape
     dt = proj.dtype
-    _need(proj.is_contiguous() and n == batch.N and wq.numel() == Rq and wkv.numel() == R and wq.dtype == dt and wkv.dtype == dt,
+    _need(proj.is_contiguous() and n == batch.N and (Rq == 0 or (wq is not None and wq.numel() == Rq and wq.dtype == dt)) and wkv.numel() == R and wkv.dtype == dt,
           "latent_prep: proj [N, ld] of the batch, norm weights over the latents")
     _need(pool.dtype == dt and pool.is_contiguous() and pool.shape[-1] == R + rd, "latent_prep: pool [tokens, R + rd]")
     tl = _angle_tables(rot_dims, cos, sin, batch, "latent_prep")
-    cq = torch.empty((n, Rq), dtype=dt, device=proj.device)
-    N.check_layers(N.layers().jl_latent_prep(_ptr(proj), _code(dt), n, ld, q_col, Rq, kv_col, R, rd, rot_dims, _ptr(wq), _ptr(wkv), float(eps),
-                                            _ptr(batch.pos), _ptr(cos), _ptr(sin), tl, _ptr(cq), _ptr(pool), _ptr(batch.kv_slot),
+    cq = torch.empty((n, Rq), dtype=dt, device=proj.device) if Rq else None
+    N.check_layers(N.layers().jl_latent_prep(_ptr(proj), _code(dt), n, ld, q_col, Rq, kv_col, R, rd, rot_dims, _ptr(wq) if Rq else None, _ptr(wkv), float(eps),
+                                            _ptr(batch.pos), _ptr(cos), _ptr(sin), tl, _ptr(cq), _ptr(pool), _ptr(batch.kv_slot), int(pairing),
                                             _stream(proj.device)), "jl_latent_prep")
     return cq
 
 
-def latent_q_pack(qa: torch.Tensor, q: torch.Tensor, H: int, D: int, R: int, rd: int, rot_dims: int, batch: RaggedBatch, cos, sin) -> torch.Tensor:
-    """qa [H, N, R] (queries times the key up-projection), q [N, H*(D + rd)] -> [N, H*(R + rd)] with the rotary part rotated."""
+def latent_q_pack(qa: torch.Tensor, q: torch.Tensor, H: int, D: int, R: int, rd: int, rot_dims: int, batch: RaggedBatch, cos, sin,
+                  pairing: int = N.JL_ROT_HALVES) -> torch.Tensor:
+    """qa [H, N, R] (queries times the key up-projection), q [N, H*(D + rd)] (row stride free: a column range of a wider product) ->
+    [N, H*(R + rd)] with the rotary part rotated."""
     _dev(q)
     n = q.shape[0]
-    _need(q.is_contiguous() and qa.is_contiguous() and tuple(qa.shape) == (H, n, R) and q.shape[1] == H * (D + rd) and qa.dtype == q.dtype and n == batch.N,
+    _need(q.stride(1) == 1 and qa.is_contiguous() and tuple(qa.shape) == (H, n, R) and q.shape[1] == H * (D + rd) and qa.dtype == q.dtype and n == batch.N,
           "latent_q_pack: qa [H, N, R], q [N, H*(D + rd)]")
     tl = _angle_tables(rot_dims, cos, sin, batch, "latent_q_pack")
     out = torch.empty((n, H * (R + rd)), dtype=q.dtype, device=q.device)
-    N.check_layers(N.layers().jl_latent_q_pack(_ptr(qa), _ptr(q), _code(q.dtype), n, H, D, R, rd, rot_dims, _ptr(batch.pos), _ptr(cos), _ptr(sin), tl,
-                                              _ptr(out), _stream(q.device)), "jl_latent_q_pack")
+    N.check_layers(N.layers().jl_latent_q_pack(_ptr(qa), _ptr(q), q.stride(0), _code(q.dtype), n, H, D, R, rd, rot_dims, _ptr(batch.pos), _ptr(cos), _ptr(sin), tl,
+                                              _ptr(out), int(pairing), _stream(q.device)), "jl_latent_q_pack")
     return out
 
 
@@ -564,4 +580,108 @@ def heads_gate(ov: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
     out = torch.empty((n, H * Dv), dtype=ov.dtype, device=ov.device)
     N.check_layers(N.layers().jl_heads_gate(_ptr(ov), _ptr(gate), gate.stride(0) if gate is not None else 0, _code(ov.dtype), n, H, Dv, _ptr(out),
                                            _stream(ov.device)), "jl_heads_gate")
+    return out
+
+
+def _addends(addends, n: int, W: int, what: str):
+    arr = (N.Addend * max(1, len(addends)))()
+    for k, (y, sc) in enumerate(addends):
+        _need(y.is_contiguous() and y.shape[0] == n and y.shape[-1] == W and y.dim() in (2, 3), f"{what}: an addend is [N, W] or [N, S, W]")
+        if sc is not None:
+            _need(sc.dtype == torch.float32 and sc.numel() == W and sc.is_contiguous(), f"{what}: a scale is float [W]")
+        arr[k] = N.Addend(y=y.data_ptr(), dtype=_code(y.dtype), count=1 if y.dim() == 2 else y.shape[1], scale=sc.data_ptr() if sc is not None else None)
+    return arr
+
+
+def depth_mix_norm(x_in: torch.Tensor, addends: Sequence[Tuple[torch.Tensor, Optional[torch.Tensor]]], mult: float, streams: Optional[torch.Tensor],
+                   depth: int, mix: Optional[torch.Tensor], x_out: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float,
+                   out_dtype: Optional[torch.dtype], want_float: bool = False):
+    """Residual update, weighted sum over the streams of all depths, RMS norm.  y = x_in + mult * sum of the addends ((tensor [N, W] or
+    [N, S, W], channel scale or None), at most three).  With ``depth`` >= 0, y becomes streams[depth] (``streams`` float [depths, N, W]) and
+    x_out = sum_{j <= depth} mix[j] * streams[j] (``mix`` float, at least depth + 1 entries; None: x_out = y); with ``depth`` < 0, x_out = y,
+    or nothing is written when there are no addends.  Returns the norm of x_out (of x_in when nothing was written) times ``w`` (float
+    [W] or None) in ``out_dtype`` — and, with ``want_float``, the same unrounded in float as a second result; None with neither."""
+    _dev(x_in)
+    n, W = x_in.shape
+    _need(x_in.dtype == torch.float32 and x_in.is_contiguous() and len(addends) <= 3, "depth_mix_norm: x_in contiguous float32 [N, W], at most 3 addends")
+    arr = _addends(addends, n, W, "depth_mix_norm")
+    written = depth >= 0 or len(addends) > 0
+    if written:
+        _need(x_out is not None and x_out.dtype == torch.float32 and x_out.is_contiguous() and x_out.shape == x_in.shape, "depth_mix_norm: x_out float [N, W]")
+    ld = 0
+    if depth >= 0:
+        _need(streams is not None and streams.dtype == torch.float32 and streams.is_contiguous() and streams.dim() == 3 and tuple(streams.shape[1:]) == (n, W) and
+              depth < streams.shape[0], "depth_mix_norm: streams float [depths, N, W] with room for this depth")
+        ld = n * W
+        if mix is not None:
+            _need(mix.dtype == torch.float32 and mix.is_contiguous() and mix.numel() >= depth + 1, "depth_mix_norm: mix float with depth + 1 entries")
+    if w is not None:
+        _need(w.dtype == torch.float32 and w.numel() == W and w.is_contiguous(), "depth_mix_norm: the norm weight is float [W]")
+    out = torch.empty((n, W), dtype=out_dtype, device=x_in.device) if out_dtype is not None else None
+    outf = torch.empty((n, W), dtype=torch.float32, device=x_in.device) if want_float else None
+    N.check_layers(N.layers().jl_depth_mix_norm(_ptr(x_in), arr, len(addends), float(mult), _ptr(streams) if depth >= 0 else None, ld, int(depth),
+                                               _ptr(mix) if depth >= 0 else None, _ptr(x_out) if written else None, _ptr(w), float(eps), _ptr(out),
+                                               _code(out_dtype or torch.float32), _ptr(outf), n, W, _stream(x_in.device)), "jl_depth_mix_norm")
+    return (out, outf) if want_float else out
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, batch: RaggedBatch, tail: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """h + (h of the previous token - h) * mu: h float [N, W], mu float [W]; ``tail`` float [slots, 1, W] carries every request's last h
+    from step to step (updated here; never read by a request that starts at position 0)."""
+    _dev(h)
+    n, W = h.shape
+    _need(h.dtype == torch.float32 and h.is_contiguous() and n == batch.N and mu.dtype == torch.float32 and mu.numel() == W and mu.is_contiguous(),
+          "token_shift: h float [N, W] of the batch, mu float [W]")
+    _need(tail.dtype == torch.float32 and tail.is_contiguous() and tail.numel() == tail.shape[0] * W and batch.max_slot < tail.shape[0],
+          "token_shift: tail float [slots, 1, W] with the batch's slots")
+    out = torch.empty((n, W), dtype=out_dtype, device=h.device)
+    N.check_layers(N.layers().jl_token_shift(_ptr(h), _ptr(mu), _ptr(batch.row_req), _ptr(batch.seq), _ptr(tail), n, W, _ptr(out), _code(out_dtype),
+                                            _stream(h.device)), "jl_token_shift")
+    return out
+
+
+def softcap(z: torch.Tensor, cap: float) -> torch.Tensor:
+    """cap * tanh(z / cap), in place on contiguous float z."""
+    _dev(z)
+    _need(z.dtype == torch.float32 and z.is_contiguous() and cap > 0, "softcap: contiguous float32 values and a positive cap")
+    N.check_layers(N.layers().jl_softcap(_ptr(z), z.numel(), float(cap), _stream(z.device)), "jl_softcap")
+    return z
+
+
+def short_conv(x: torch.Tensor, col: int, C_: int, w: torch.Tensor, batch: RaggedBatch, tail: Optional[torch.Tensor], act: int = N.JL_ACT_SILU) -> torch.Tensor:
+    """act(causal depthwise convolution over time, per request) of the columns col .. col + C_ of x [N, ld], with w [C_, taps]; float
+    [N, C_].  ``tail`` float [slots, taps - 1, C_] carries every request's last inputs from step to step (updated here)."""
+    _dev(x)
+    n, ld = x.shape
+    taps = w.shape[1]
+    _need(x.is_contiguous() and n == batch.N and w.is_contiguous() and w.shape[0] == C_ and w.dtype == x.dtype and 0 <= col and col + C_ <= ld and 1 <= taps <= 8,
+          "short_conv: x [N, ld] of the batch, w [C, taps <= 8] of its dtype, the columns inside the row")
+    if taps > 1:
+        _need(tail is not None and tail.dtype == torch.float32 and tail.is_contiguous() and tuple(tail.shape[1:]) == (taps - 1, C_) and
+              batch.max_slot < tail.shape[0], "short_conv: tail float [slots, taps - 1, C] with the batch's slots")
+    out = torch.empty((n, C_), dtype=torch.float32, device=x.device)
+    N.check_layers(N.layers().jl_short_conv(_ptr(x), _code(x.dtype), ld, col, _ptr(w), _ptr(batch.row_req), _ptr(batch.seq), batch.B, max(batch.counts),
+                                           _ptr(tail), n, C_, taps, int(act), _ptr(out), _stream(x.device)), "jl_short_conv")
+    return out
+
+
+def delta_rule(qkv: torch.Tensor, cols: Tuple[int, int, int], proj: torch.Tensor, pcols: Tuple[int, int, int], a_log: torch.Tensor, dt_bias: torch.Tensor,
+               norm_w: torch.Tensor, batch: RaggedBatch, H: int, G: int, D: int, Dv: int, unit_eps: float, q_scale: float, eps: float,
+               state: torch.Tensor) -> torch.Tensor:
+    """Gated delta rule.  qkv float [N, *] holds q, k (G*D each) and v (H*Dv) at ``cols`` (after convolution and activation); proj [N, ld]
+    holds the decay input a, the step input b (H each) and the gate (H*Dv) at ``pcols``; a_log, dt_bias float [H]; norm_w float [Dv];
+    state [slots, H, D, Dv] float (updated in place).  Returns [N, H*Dv] of proj's dtype."""
+    _dev(proj)
+    n, ld = proj.shape
+    _need(proj.is_contiguous() and n == batch.N and qkv.dtype == torch.float32 and qkv.is_contiguous() and qkv.shape[0] == n, "delta_rule: proj and float qkv of the batch")
+    _need(H % G == 0 and max(cols[0], cols[1]) + G * D <= qkv.shape[1] and cols[2] + H * Dv <= qkv.shape[1] and max(pcols[0], pcols[1]) + H <= ld and
+          pcols[2] + H * Dv <= ld, "delta_rule: columns do not fit the rows")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv) and batch.max_slot < state.shape[0],
+          "delta_rule: state float [slots, H, D, Dv] with the batch's slots")
+    for t, k in ((a_log, H), (dt_bias, H), (norm_w, Dv)):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == k, "delta_rule: a_log, dt_bias float [H], norm_w float [Dv]")
+    out = torch.empty((n, H * Dv), dtype=proj.dtype, device=proj.device)
+    N.check_layers(N.layers().jl_delta_rule(_ptr(qkv), N.JL_F32, qkv.shape[1], cols[0], cols[1], cols[2], _ptr(proj), _code(proj.dtype), ld, pcols[0], pcols[1],
+                                           pcols[2], _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), _ptr(batch.seq), batch.B, H, G, D, Dv, float(unit_eps),
+                                           float(q_scale), float(eps), _ptr(state), _ptr(out), _stream(proj.device)), "jl_delta_rule")
     return out

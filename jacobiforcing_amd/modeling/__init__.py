@@ -15,6 +15,7 @@ MODEL_REGISTRY = {
     "Lokizen": ("jacobiforcing_amd.modeling.lokizen", "LokizenConfig", "ragged"),
     "Vumalix": ("jacobiforcing_amd.modeling.vumalix", "VumalixConfig", "ragged"),
     "Bamanex": ("jacobiforcing_amd.modeling.bamanex", "BamanexConfig", "ragged"),
+    "Mikipel": ("jacobiforcing_amd.modeling.mikipel", "MikipelConfig", "ragged"),
 }
 
 
