@@ -730,7 +730,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=96)
-    ap.add_argument("--design", default="", help="'lokizen' / 'vumalix' / 'bamanex': instead of the default workload, prefill / decode throughput of that ragged "
+    ap.add_argument("--design", default="", help="'lokizen' / 'vumalix' / 'bamanex' / 'mikipel': instead of the default workload, prefill / decode throughput of that ragged "
                     "family at real-layer sizes beside the closest existing model at equal size, and each layer kernel against its roofline (one JSON line)")
     ap.add_argument("--design-sizes", default="small,medium")
     ap.add_argument("--warmup", type=int, default=16)
@@ -755,8 +755,8 @@ def main():
     if args.gpus < 1:
         raise SystemExit("--gpus must be >= 1")
     if args.design:
-        if args.design.lower() not in ("lokizen", "vumalix", "bamanex"):
-            raise SystemExit(f"--design {args.design}: only 'lokizen', 'vumalix' and 'bamanex' have a comparison section")
+        if args.design.lower() not in ("lokizen", "vumalix", "bamanex", "mikipel"):
+            raise SystemExit(f"--design {args.design}: only 'lokizen', 'vumalix', 'bamanex' and 'mikipel' have a comparison section")
         if not torch.cuda.is_available():
             raise SystemExit("bench.py needs an MI355X: the layer kernels have no CPU path")
         from jacobiforcing_amd.drivers import ragged_bench

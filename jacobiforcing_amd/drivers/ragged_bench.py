@@ -1,9 +1,9 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of a ragged model family (Lokizen, Vumalix, Bamanex) at sizes that resemble a real model's layers,
-beside the package's closest existing model at equal width, depth, head sizes and active feed-forward width (Lokizen beside Qwen2;
-Vumalix beside Lokizen and Qwen2; Bamanex beside Lokizen and Qwen2) — random weights, synthetic tokens.
+"""Prefill and decode throughput of a ragged model family (Lokizen, Vumalix, Bamanex, Mikipel) at sizes that resemble a real model's
+layers, beside the package's closest existing model at equal width, depth, head sizes and active feed-forward width (Lokizen beside
+Qwen2; Vumalix, Bamanex and Mikipel beside Lokizen and Qwen2) — random weights, synthetic tokens.
 
-    python -m jacobiforcing_amd.drivers.ragged_bench [--design lokizen|vumalix|bamanex] [--sizes small,medium] [--kernels]
+    python -m jacobiforcing_amd.drivers.ragged_bench [--design lokizen|vumalix|bamanex|mikipel] [--sizes small,medium] [--kernels]
     python bench.py --design lokizen            (the same, as one JSON line)
 
 Per size: prefill = whole prompts in one step (tokens / s), decode = one token for each of ``--decode-batch`` requests at a
@@ -399,6 +399,158 @@ def kernel_table_bamanex(s, prompts, prompt_len, decode_batch, context, dtype=to
     return out
 
 
+# Mikipel at Lokizen's widths, depths, head counts, head sizes and experts: the delta rule where Lokizen has retention, grouped-query
+# attention and latent attention (Vumalix's latent sizes) taking turns where it has windowed attention; one dense feed-forward of the
+# experts' active width, experts elsewhere; four taps
+def mikipel_config(s):
+    from ..modeling.mikipel import MikipelConfig
+    H, G, D, W = s["heads"], s["kv"], s["dim"], s["width"]
+    v = VSIZES["small" if W <= 1024 else "medium"]
+    moe = {"kind": "moe", "expert": {"ff": s["ff"]}, "router": {"experts": s["experts"], "top": s["top"]}}
+    dense = {"kind": "dense", "ff": s["top"] * s["ff"]}
+    dlt = {"type": "delta", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "conv": 4}}
+    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "rot": {"dims": D, "base": 1e6, "scaling": {"factor": 8.0}}}}
+    lat = {"type": "latent_attention", "mixer": {"heads": v["lheads"], "dim": v["ldim"], "rot_dim": v["rot"], "vdim": v["lvdim"], "kv_rank": v["kv_rank"],
+                                                 "scale": (v["ldim"] + v["rot"]) ** -0.5, "rot": {"dims": v["rot"], "base": 1e6}}}
+    order = [dlt, att, dlt, lat]
+    return MikipelConfig.from_dict({"architecture": "Mikipel", "vocab": s["vocab"], "width": W, "norm": {"eps": 1e-6}, "embedding": {"scale": W ** 0.5},
+                                    "residual_mult": 0.3, "logit_softcap": 30.0,
+                                    "layers": [dict(order[i % 4], mlp=dense if i == 1 else moe) for i in range(s["layers"])]})
+
+
+def bench_mikipel(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
+    from ..modeling.mikipel import random_model
+    model = random_model(mikipel_config(s), "cuda", dtype, max_positions=max(prompt_len, context) + 64)
+    return bench_ragged(model, s["vocab"], prompts, prompt_len, decode_batch, context)
+
+
+def kernel_table_mikipel(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
+    """Mikipel's layer kernels alone at the size's shapes, prefill and decode, each beside the like kernel of the closest model
+    (Lokizen's residual + norm launch, its retention scan, its windowed attention, its routed experts; Vumalix's convolution; Qwen2's
+    SwiGLU launch)."""
+    from .. import layer_ops as LO
+    from .. import ops
+    dev = "cuda"
+    H, G, D, W, E, top, ff, win, L = s["heads"], s["kv"], s["dim"], s["width"], s["experts"], s["top"], s["ff"], s["window"], s["layers"]
+    page, es = 64, 2
+    per = -(-(max(prompt_len, context) + 1) // page)
+    slots = max(prompts, decode_batch)
+    tables = [list(range(b * per, (b + 1) * per)) for b in range(slots)]
+    g = torch.Generator().manual_seed(0)
+    rnd = lambda *sh: torch.randn(*sh, generator=g).to(dev).to(dtype)
+    kc, vc = rnd(slots * per * page, G * D), rnd(slots * per * page, G * D)
+    a = torch.arange(max(prompt_len, context) + 8, dtype=torch.float32, device=dev).view(-1, 1) * torch.rand(D // 2, device=dev).view(1, -1)
+    cos, sin = a.cos().contiguous(), a.sin().contiguous()
+    state, decay = torch.zeros((slots, H, D, D), device=dev), torch.full((H,), 0.99, device=dev)
+    a_log, dt_bias, nw = torch.zeros(H, device=dev), torch.zeros(H, device=dev), torch.ones(D, device=dev)
+    C_ = 2 * G * D + H * D
+    taps = 4
+    ctail, stail, vtail = torch.zeros((slots, taps - 1, C_), device=dev), torch.zeros((slots, 1, W), device=dev), torch.zeros((slots, taps - 1, W), device=dev)
+    w_gu, w_up, w_down = rnd(E, 2 * ff, W) * 0.02, rnd(E, ff, W) * 0.02, rnd(E, W, ff) * 0.02
+    out = {}
+
+    def row(name, secs, nbytes, flops, peak):
+        bound = max(nbytes / HBM_BPS, flops / peak)
+        out[name] = {"us": round(1e6 * secs, 1), "MB": round(nbytes / 1e6, 2), "GFLOP": round(flops / 1e9, 2), "roofline_fraction": round(bound / secs, 4)}
+
+    for phase, B, T, start in (("prefill", prompts, prompt_len, 0), ("decode", decode_batch, 1, context)):
+        n = B * T
+        batch = LO.RaggedBatch.build([T] * B, [start] * B, list(range(B)), tables[:B], page, dev)
+        causal = B * sum(start + t + 1 for t in range(T))                                       # visible (query, key) pairs per head
+        windowed = B * sum(min(start + t + 1, win) for t in range(T))
+        span_c, span_w = B * (start + T), B * min(start + T, win + T)                              # pool rows a launch has to read once
+        # residual sum + mixture of the depths + norm (rounded and unrounded), at half depth and at full depth  |  Lokizen: one addend, one norm
+        x, y1, y2, wn = torch.randn(n, W, device=dev), rnd(n, W), torch.randn(n, top, W, device=dev), torch.randn(W, device=dev)
+        streams, mix, xo = torch.randn(L + 1, n, W, device=dev), torch.randn(L + 1, device=dev), torch.empty(n, W, device=dev)
+        for d in (L // 2, L):
+            row(f"{phase}.depth_mix_norm(depth {d})", timed(lambda: LO.depth_mix_norm(x, [(y1, None), (y2, None)], 0.3, streams, d, mix, xo, wn, 1e-6, dtype, want_float=True)),
+                n * W * (4 + es + 4 * top + 4 + 4 * d + 4 + 4 + es + 4), (2.0 * d + 10) * n * W, VECTOR_FLOPS)
+        row(f"{phase}.lokizen.add_rmsnorm", timed(lambda: LO.add_rmsnorm(x, y2, None, wn.to(dtype), 1e-5, dtype)), n * W * (4 + 4 * top + 4 + 4 + es), 4.0 * n * W, VECTOR_FLOPS)
+        hf = torch.randn(n, W, device=dev)
+        row(f"{phase}.token_shift", timed(lambda: LO.token_shift(hf, wn, batch, stail, dtype)), n * W * (4 + es), 3.0 * n * W, VECTOR_FLOPS)
+        # short convolution + silu of q | k | v  |  Vumalix: convolution of the stream, added to it
+        proj = rnd(n, C_ + H * D + 2 * H + (-(C_ + H * D + 2 * H)) % 8)
+        cw = rnd(C_, taps)
+        row(f"{phase}.short_conv(silu)", timed(lambda: LO.short_conv(proj, 0, C_, cw, batch, ctail, LO.ACT_SILU)), n * C_ * (es + 4), (2.0 * taps + 4) * n * C_, VECTOR_FLOPS)
+        vw = rnd(W, taps)
+        row(f"{phase}.vumalix.causal_conv", timed(lambda: LO.causal_conv(x, vw, batch, vtail)), n * W * (4 + es), 2.0 * taps * n * W, VECTOR_FLOPS)
+        # gated delta rule  |  Lokizen: retention (fixed decay, no correction term)
+        qkv = LO.short_conv(proj, 0, C_, cw, batch, ctail, LO.ACT_SILU)
+        t_dl = timed(lambda: LO.delta_rule(qkv, (0, G * D, 2 * G * D), proj, (C_ + H * D, C_ + H * D + H, C_), a_log, dt_bias, nw, batch, H, G, D, D, 1e-6, D ** -0.5, 1e-6, state))
+        row(f"{phase}.delta_rule", t_dl, n * (C_ * 4 + (2 * H * D + 2 * H) * es) + 2 * B * H * D * D * 4, 6.0 * n * H * D * D, VECTOR_FLOPS)
+        pr = rnd(n, 4 * H * D)
+        t_ret = timed(lambda: LO.retention(pr, (0, H * D, 2 * H * D, 3 * H * D), batch, H, D, D, D, cos, sin, decay, 1e-5, state))
+        row(f"{phase}.lokizen.retention", t_ret, n * 5 * H * D * es + 2 * B * H * D * D * 4, 4.0 * n * H * D * D, VECTOR_FLOPS)
+        # plain causal grouped-query attention (rotation + unit norm + append, then the one-sweep kernel)  |  Lokizen: windowed attention
+        pa = rnd(n, H * D + 2 * G * D)
+        cols = (0, H * D, H * D + G * D)
+        t_hn = timed(lambda: LO.head_norm_append(pa, cols, H, G, 1, D, D, None, None, 1e-6, 0.0, 1, batch, kc, vc, rot_dims=D, cos=cos, sin=sin))
+        row(f"{phase}.head_norm_append(rot)", t_hn, 2 * n * (H * D + 2 * G * D) * es, 10.0 * n * (H + G) * D, VECTOR_FLOPS)
+        q = LO.head_norm_append(pa, cols, H, G, 1, D, D, None, None, 1e-6, 0.0, 1, batch, kc, vc, rot_dims=D, cos=cos, sin=sin)
+        sweep = LO.attn_sweep_tile_rows(dtype, H, G, D, D, kc, vc) > 0
+        t_at = timed(lambda: LO.attn_sweep(q, kc, vc, batch, H, G, D, D, D ** -0.5, 0) if sweep else LO.attn_window(q, None, kc, vc, batch, H, G, D, D, D ** -0.5, 0, 0, None, None, None))
+        row(f"{phase}.attn_causal", t_at, span_c * 2 * G * D * es + 2 * n * H * D * es, 4.0 * causal * H * D, MATRIX_FLOPS)
+        gate = rnd(n, H * D)
+        rel, talk = torch.randn(max(prompt_len, context) + 8, H, device=dev), torch.eye(H, device=dev)
+        t_lw = timed(lambda: LO.attn_window(q, gate, kc, vc, batch, H, G, D, D, D ** -0.5, win, 4, rel, None, talk))
+        row(f"{phase}.lokizen.attn_window", t_lw, span_w * 2 * G * D * es + 3 * n * H * D * es, 4.0 * windowed * H * D, MATRIX_FLOPS)
+        # latent attention without a query latent, neighbouring rotation pairs, no window
+        v = VSIZES["small" if W <= 1024 else "medium"]
+        LH, LD, rd, LDv, R = v["lheads"], v["ldim"], v["rot"], v["lvdim"], v["kv_rank"]
+        lat = rnd(slots * per * page, R + rd)
+        pl = rnd(n, LH * (LD + rd) + R + rd)
+        wlk = rnd(R)
+        al = torch.arange(max(prompt_len, context) + 8, dtype=torch.float32, device=dev).view(-1, 1) * torch.rand(rd // 2, device=dev).view(1, -1)
+        lc, ls_ = al.cos().contiguous(), al.sin().contiguous()
+        t_lp = timed(lambda: LO.latent_prep(pl, 0, 0, LH * (LD + rd), R, rd, rd, None, wlk, 1e-6, batch, lc, ls_, lat, pairing=LO.ROT_NEIGHBOURS))
+        row(f"{phase}.latent_prep", t_lp, 2 * n * (R + rd) * es, 6.0 * n * (R + rd), VECTOR_FLOPS)
+        qa, ql = rnd(LH, n, R), pl[:, :LH * (LD + rd)]
+        row(f"{phase}.latent_q_pack", timed(lambda: LO.latent_q_pack(qa, ql, LH, LD, R, rd, rd, batch, lc, ls_, pairing=LO.ROT_NEIGHBOURS)), 2 * n * LH * (R + rd) * es,
+            6.0 * n * LH * rd, VECTOR_FLOPS)
+        qf = LO.latent_q_pack(qa, ql, LH, LD, R, rd, rd, batch, lc, ls_, pairing=LO.ROT_NEIGHBOURS)
+        step = LO.ATTN_MAX_VALUE_WIDTH
+
+        def latent_attn():
+            if LO.attn_sweep_tile_rows(dtype, LH, 1, R + rd, R, lat, lat[:, :R]):
+                return LO.attn_sweep(qf, lat, lat[:, :R], batch, LH, 1, R + rd, R, 0.1, 0)
+            return [LO.attn_window(qf, None, lat, lat[:, c0:min(R, c0 + step)], batch, LH, 1, R + rd, min(R, c0 + step) - c0, 0.1, 0, 0, None, None, None)
+                    for c0 in range(0, R, step)]
+        row(f"{phase}.attn_latent", timed(latent_attn), span_c * (R + rd) * es + n * LH * (2 * R + rd) * es, 2.0 * causal * LH * (2 * R + rd), MATRIX_FLOPS)
+        # activations  |  Qwen2's SwiGLU launch
+        up = rnd(n, top * ff)
+        row(f"{phase}.gated_act(gelu_erf, no linear branch)", timed(lambda: LO.gated_act(up, 0, -1, top * ff, LO.ACT_GELU_ERF)), 2 * n * top * ff * es, 10.0 * n * top * ff, VECTOR_FLOPS)
+        gu = rnd(n, 2 * top * ff)
+        row(f"{phase}.qwen2.swiglu", timed(lambda: ops.swiglu(gu)), 3 * n * top * ff * es, 4.0 * n * top * ff, VECTOR_FLOPS)
+        # routed experts: silu units, softmax over the chosen logits  |  Lokizen: relu^2 units, sigmoid routing
+        h, z = rnd(n, W), torch.randn(n, E, device=dev)
+        used = min(E, n * top)
+        t_moe = timed(lambda: LO.moe_experts(h, z, None, top, 1.0, w_gu, w_down, route="top_softmax", gated=(LO.ACT_SILU, 0.0, 1.0, 0.0)))
+        row(f"{phase}.moe_experts(silu units)", t_moe, used * 3 * ff * W * es + n * W * es + n * top * W * 4, 6.0 * n * top * ff * W, MATRIX_FLOPS)
+        t_moe = timed(lambda: LO.moe_experts(h, z, None, top, 1.0, w_up, w_down))
+        row(f"{phase}.lokizen.moe_experts", t_moe, used * 2 * ff * W * es + n * W * es + n * top * W * 4, 4.0 * n * top * ff * W, MATRIX_FLOPS)
+        zl = torch.randn(B, s["vocab"], device=dev)
+        row(f"{phase}.softcap", timed(lambda: LO.softcap(zl, 30.0)), 2 * B * s["vocab"] * 4, 8.0 * B * s["vocab"], VECTOR_FLOPS)
+    return out
+
+
+def run_mikipel(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True):
+    res = {"bench": "ragged_family", "design": "Mikipel", "closest": "Lokizen", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
+           "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
+    for name in sizes:
+        s = SIZES[name]
+        entry = {"shape": s, "mikipel": bench_mikipel(s, prompts, prompt_len, decode_batch, context)}
+        torch.cuda.empty_cache()
+        entry["lokizen"] = bench_lokizen(s, prompts, prompt_len, decode_batch, context)
+        torch.cuda.empty_cache()
+        entry["qwen2"] = bench_qwen2(s, prompts, prompt_len, decode_batch, context)
+        torch.cuda.empty_cache()
+        if kernels:
+            entry["kernels"] = kernel_table_mikipel(s, prompts, prompt_len, decode_batch, context)
+            torch.cuda.empty_cache()
+        res["sizes"][name] = entry
+    return res
+
+
 def run_bamanex(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True):
     res = {"bench": "ragged_family", "design": "Bamanex", "closest": "Lokizen", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
            "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
@@ -440,6 +592,8 @@ def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, 
         return run_vumalix(sizes, prompts, prompt_len, decode_batch, context, kernels)
     if design.lower() == "bamanex":
         return run_bamanex(sizes, prompts, prompt_len, decode_batch, context, kernels)
+    if design.lower() == "mikipel":
+        return run_mikipel(sizes, prompts, prompt_len, decode_batch, context, kernels)
     res = {"bench": "ragged_family", "design": "Lokizen", "closest": "Qwen2", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
            "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
     for name in sizes:
@@ -457,7 +611,7 @@ def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
-    ap.add_argument("--design", default="lokizen", choices=("lokizen", "vumalix", "bamanex"))
+    ap.add_argument("--design", default="lokizen", choices=("lokizen", "vumalix", "bamanex", "mikipel"))
     ap.add_argument("--sizes", default="small,medium")
     ap.add_argument("--prompts", type=int, default=4)
     ap.add_argument("--prompt-len", type=int, default=2048)
