@@ -17,7 +17,7 @@ extern "C" {
 #endif
 
 #define JL_API __attribute__((visibility("default")))
-#define JL_VERSION 122
+#define JL_VERSION 123
 #define JL_OK 0
 #define JL_E_INVALID (-1)
 #define JL_E_LAUNCH (-3)
@@ -241,11 +241,14 @@ JL_API int jl_retention_join(const int32_t *req, int32_t B, const int32_t *chunk
  *   out_h(t) = o / sqrt(mean(o^2) + eps) * norm_w * silu(gate_h(t))             (norm_w float [Dv], shared by the heads)
  * qkv float [N, qkv_ld] holds q, k (G*D columns each) and v (H*Dv) after their convolution and activation; proj [N, ld] of `dtype` holds
  * a, b (H columns each) and the gate (H*Dv).  state [slots, H, D, Dv] float: a request with pos0 == 0 starts from zero (its slot's old
- * content is ignored); the final state is written back.  out [N, H*Dv] of `dtype`.  D <= 256, Dv <= 1024. */
+ * content is ignored); the final state is written back.  out [N, H*Dv] of `dtype`, N the batch's rows.  D <= 256, Dv <= 1024.
+ * `raw` null: one workgroup per (request, head) that also normalises and gates (single tokens, short portions).  `raw` = N * H * Dv floats
+ * of scratch: the form for long portions — the state's columns shared out over single-wavefront workgroups whose unnormalised outputs go
+ * to `raw`, and a second launch for norm and gate. */
 JL_API int jl_delta_rule(const void *qkv, int qkv_dtype, int64_t qkv_ld, int32_t q_col, int32_t k_col, int32_t v_col, const void *proj, int dtype,
                          int64_t ld, int32_t a_col, int32_t b_col, int32_t g_col, const float *A_log, const float *dt_bias, const float *norm_w,
-                         const int32_t *seq, int32_t B, int32_t H, int32_t G, int32_t D, int32_t Dv, float unit_eps, float q_scale, float eps,
-                         float *state, void *out, void *stream);
+                         const int32_t *seq, int32_t B, int64_t N, int32_t H, int32_t G, int32_t D, int32_t Dv, float unit_eps, float q_scale, float eps,
+                         float *state, float *raw, void *out, void *stream);
 
 /* Router of a mixture of experts over float logits [N, E]; ids [N, top] int32, weights [N, top] float.
  *   JL_ROUTE_SIGMOID:        s = sigmoid(logits); the `top` experts with the largest s + correction are chosen (ties: lowest

@@ -21,6 +21,7 @@ ATTN_MAX_HEADS_ONE_LAUNCH, ATTN_MAX_VALUE_WIDTH = 16, 128   # what the matrix-co
 SWEEP_SPLIT_BELOW_GROUPS, SWEEP_SPLIT_WORKGROUPS = 512, 2048   # one-sweep attention: its workgroups are small (4 wavefronts, <= 32 rows)
 SWEEP_WIDE_ROWS_PER_REQUEST = 16   # one-sweep attention: from this many tokens per request on average a step takes the 128-row tiles
 RETENTION_CHUNK = 64          # tokens per chunk when a long portion's recurrence is cut into chunks that run side by side
+DELTA_COLUMNS_FROM = 32       # delta rule: from this many tokens in a request's portion on, the state's columns are shared out over wavefronts
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -681,7 +682,9 @@ def delta_rule(qkv: torch.Tensor, cols: Tuple[int, int, int], proj: torch.Tensor
     for t, k in ((a_log, H), (dt_bias, H), (norm_w, Dv)):
         _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() == k, "delta_rule: a_log, dt_bias float [H], norm_w float [Dv]")
     out = torch.empty((n, H * Dv), dtype=proj.dtype, device=proj.device)
+    long_portions = max(batch.counts) >= DELTA_COLUMNS_FROM and not os.environ.get("JL_DELTA_NO_COLUMNS")          # A/B switch for measurements
+    raw = torch.empty((n, H * Dv), dtype=torch.float32, device=proj.device) if long_portions else None
     N.check_layers(N.layers().jl_delta_rule(_ptr(qkv), N.JL_F32, qkv.shape[1], cols[0], cols[1], cols[2], _ptr(proj), _code(proj.dtype), ld, pcols[0], pcols[1],
-                                           pcols[2], _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), _ptr(batch.seq), batch.B, H, G, D, Dv, float(unit_eps),
-                                           float(q_scale), float(eps), _ptr(state), _ptr(out), _stream(proj.device)), "jl_delta_rule")
+                                           pcols[2], _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), _ptr(batch.seq), batch.B, n, H, G, D, Dv, float(unit_eps),
+                                           float(q_scale), float(eps), _ptr(state), _ptr(raw), _ptr(out), _stream(proj.device)), "jl_delta_rule")
     return out

@@ -391,8 +391,9 @@ MIXER_SIZES = [attn(4, 2, 32, 64, 16), attn(8, 8, 64, 32, 64, factor=0.0), attn(
 @pytest.mark.parametrize("layer", MIXER_SIZES, ids=lambda L: L["type"][0] + "-".join(str(v) for v in L["mixer"].values() if not isinstance(v, (dict, float))))
 def test_each_mixer_alone_in_portions_and_single_tokens(layer):
     """One mixer on the oracle's own inputs, float32 and bfloat16: a prompt's first part in one step, a second part that starts inside a
-    page and inside a group of the recurrence, two tokens, then single tokens, on shuffled pages and a poisoned slot."""
-    W, T = 64, 43
+    page and inside a group of the recurrence, two tokens, then single tokens, then a long portion (the recurrence's form with the state's
+    columns shared out), on shuffled pages and a poisoned slot."""
+    W, T = 64, 84
     cfg = make_cfg([dict(layer, mlp=None)], width=W, vocab=40)
     t = tensors_for(cfg, 5)
     P = layer_tensors(t, 0)
@@ -405,7 +406,7 @@ def test_each_mixer_alone_in_portions_and_single_tokens(layer):
         want = O.MIXERS[kind](hd.cpu().double(), P, layer["mixer"], 1e-5)
         run = {"attention": rig.model._attention, "latent_attention": rig.model._latent_attention, "delta": rig.model._delta}[kind]
         got, at = [], 0
-        for n in (19, 14, 2, 1, 1, 1, 5):
+        for n in (19, 14, 2, 1, 1, 1, 5, 41):
             b, _ = rig.batch([("r", [0] * n)])
             got.append(torch.nn.functional.linear(run(0, hd[at:at + n].contiguous(), b, rig.cache), rig.model.w.layers[0]["w_o"]).float().cpu())
             at += n
@@ -637,7 +638,7 @@ def test_random_configurations_in_a_mixed_schedule(seed):
         step = []
         for k, s in seqs.items():
             if at[k] < len(s) and r.random() < 0.8:
-                n = min(len(s) - at[k], r.choice([1, 1, 2, 3, 7, 8, 9, 20]))
+                n = min(len(s) - at[k], r.choice([1, 1, 2, 3, 7, 8, 9, 20, 40]))
                 step.append((k, at[k], n)); at[k] += n
         if step:
             plan.append(step)
