@@ -17,7 +17,7 @@ extern "C" {
 #endif
 
 #define JL_API __attribute__((visibility("default")))
-#define JL_VERSION 123
+#define JL_VERSION 124
 #define JL_OK 0
 #define JL_E_INVALID (-1)
 #define JL_E_LAUNCH (-3)
@@ -126,10 +126,13 @@ JL_API int jl_attn_sweep_wide_tile_rows(int dtype, int32_t H, int32_t G, int32_t
  *   depth >= 0:  streams[depth][n] = y[n];  x_out[n] = sum_{j <= depth} mix[j] * streams[j][n]   (mix null: x_out = y)
  *   depth <  0:  x_out[n] = y[n]              (no addends: nothing is stored, the norm reads x_in)
  *   out[n] = x_out[n] / sqrt(mean(x_out[n]^2) + eps) * w     in `dtype`, and / or unrounded in out_f32 (either may be null; w null = 1)
- * streams: float, stream j at streams + j * stream_ld.  x_out may be x_in but must not lie inside streams[0 .. depth]. */
+ * streams: float, stream j at streams + j * stream_ld.  x_out may be x_in but must not lie inside streams[0 .. depth].
+ * With shift_mu (float [W]) the launch also does jl_token_shift's work, for a step in which EVERY request brings one row (N = B, row n is
+ * request n of seq [B, 4]): out_shift[n] = h + (tail[slot] - h) * shift_mu with h the unrounded norm (no tail before position 0), and
+ * tail[slot] = h. */
 JL_API int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, int32_t n_addends, float mult, float *streams, int64_t stream_ld,
                              int32_t depth, const float *mix, float *x_out, const float *w, float eps, void *out, int dtype, float *out_f32,
-                             int64_t N, int32_t W, void *stream);
+                             int64_t N, int32_t W, const float *shift_mu, const int32_t *seq, float *shift_tail, void *out_shift, void *stream);
 
 /* Token shift: out[t] = h[t] + (h[t-1] - h[t]) * mu, element by element, h float [N, W], mu float [W], out [N, W] of `dtype`.  h[t-1] of
  * a request's first row is tail[slot] (float [slots, W]) when the request has a past (pos0 > 0) and zero otherwise; tail[slot] then

@@ -231,7 +231,7 @@ def raise_state_error(code: int, what: str, aux: int = 0):
 
 # ---- libjf_layers.so (include/jf_layers.h): layer kernels of the models whose forward is not stock PyTorch ----------------------------
 JL_F32, JL_BF16 = 0, 1
-JL_VERSION = 123                 # include/jf_layers.h: a library of another version is not called (its signatures may differ)
+JL_VERSION = 124                 # include/jf_layers.h: a library of another version is not called (its signatures may differ)
 JL_OUT_SAME, JL_OUT_F32 = 0, 2
 JL_ACT_GELU_TANH, JL_ACT_CLAMPED_SWISH, JL_ACT_SILU, JL_ACT_GELU_ERF, JL_ACT_NONE = 0, 1, 2, 3, -1
 JL_ROUTE_SIGMOID, JL_ROUTE_SOFTMAX_RENORM, JL_ROUTE_TOP_SOFTMAX = 0, 1, 2
@@ -279,7 +279,8 @@ _LAYER_SIGNATURES = {
     "jl_latent_prep": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _vp, _vp,
                                  _vp, _i32, _vp]),
     "jl_latent_q_pack": (C.c_int, [_vp, _vp, _i64, C.c_int, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp, _i32, _vp]),
-    "jl_depth_mix_norm": (C.c_int, [_vp, C.POINTER(Addend), _i32, _f32, _vp, _i64, _i32, _vp, _vp, _vp, _f32, _vp, C.c_int, _vp, _i64, _i32, _vp]),
+    "jl_depth_mix_norm": (C.c_int, [_vp, C.POINTER(Addend), _i32, _f32, _vp, _i64, _i32, _vp, _vp, _vp, _f32, _vp, C.c_int, _vp, _i64, _i32, _vp, _vp, _vp, _vp,
+                                    _vp]),
     "jl_token_shift": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _vp, C.c_int, _vp]),
     "jl_softcap": (C.c_int, [_vp, _i64, _f32, _vp]),
     "jl_short_conv": (C.c_int, [_vp, C.c_int, _i64, _i32, _vp, _vp, _vp, _i32, _i32, _vp, _i64, _i32, _i32, _i32, _vp, _vp]),

@@ -251,7 +251,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void depth_mix_norm_kernel(const float *__restrict__ x_in, jl_addend a0, jl_addend a1, jl_addend a2, float mult,
                                                               float *__restrict__ streams, int64_t stream_ld, int depth, const float *__restrict__ mix,
                                                               float *__restrict__ x_out, const float *__restrict__ w, float eps, T *__restrict__ out,
-                                                              float *__restrict__ out_f32, int W) {
+                                                              float *__restrict__ out_f32, int W, const float *__restrict__ shift_mu,
+                                                              const int32_t *__restrict__ seq, float *shift_tail, T *__restrict__ out_shift) {
     __shared__ float red[16];
     const int64_t n = blockIdx.x;
     const jl_addend ad[3] = {a0, a1, a2};
@@ -277,21 +278,33 @@ __global__ __launch_bounds__(256) void depth_mix_norm_kernel(const float *__rest
         if (update) x_out[n * W + c] = v;
         ss += v * v;
     }
-    if (!out && !out_f32) return;
+    if (!out && !out_f32 && !shift_mu) return;
     ss = block_sum_f32(ss, red);
     const float r = 1.0f / sqrtf(ss / (float)W + eps);
     const float *xr = update ? x_out + n * W : x_in + n * W;
+    // the token shift in the same launch, for steps in which every request brings ONE row (row n is request n): the previous token's
+    // norm is the slot's tail (nothing before position 0), which this thread then replaces by its own
+    int slot = 0;
+    bool past = false;
+    if (shift_mu) { slot = seq[4 * n + 3]; past = seq[4 * n + 2] > 0; }
     for (int c = threadIdx.x; c < W; c += 256) {
         const float v = xr[c] * r * (w ? w[c] : 1.0f);
         if (out) st_f(out + n * W + c, v);
         if (out_f32) out_f32[n * W + c] = v;
+        if (shift_mu) {
+            float *tl = shift_tail + (int64_t)slot * W + c;
+            const float prev = past ? *tl : 0.f;
+            *tl = v;
+            st_f(out_shift + n * W + c, v + (prev - v) * shift_mu[c]);
+        }
     }
 }
 
 extern "C" int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, int32_t n_addends, float mult, float *streams, int64_t stream_ld,
                                  int32_t depth, const float *mix, float *x_out, const float *w, float eps, void *out, int dtype, float *out_f32,
-                                 int64_t N, int32_t W, void *stream) {
+                                 int64_t N, int32_t W, const float *shift_mu, const int32_t *seq, float *shift_tail, void *out_shift, void *stream) {
     if (N <= 0) return JL_OK;
+    if (shift_mu && (!seq || !shift_tail || !out_shift)) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: the token shift needs seq, tail and an output");
     if (!x_in || W <= 0 || n_addends < 0 || n_addends > 3 || (n_addends && !addends))
         return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: null pointer, bad width or more than 3 addends");
     if ((depth >= 0 || n_addends) && !x_out) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: an updated stream needs x_out");
@@ -304,7 +317,8 @@ extern "C" int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, in
         if (ad[k].y && ad[k].count <= 0) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: addend %d has no rows", k);
     }
     JL_DISPATCH(dtype, depth_mix_norm_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x_in, ad[0], ad[1], ad[2], mult, streams, stream_ld, depth,
-                                                                                                    mix, x_out, w, eps, (T *)out, out_f32, W));
+                                                                                                    mix, x_out, w, eps, (T *)out, out_f32, W, shift_mu, seq,
+                                                                                                    shift_tail, (T *)out_shift));
     return jl_check_launch("depth_mix_norm_kernel");
 }
 

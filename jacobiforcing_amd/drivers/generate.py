@@ -6,7 +6,7 @@
     python -m jacobiforcing_amd.drivers.generate --model DIR --synthetic 8 --prompt-len 200 --temperature 0.8
 
 ``prompts.json`` holds a list of token-id lists (or of strings, when the directory has a tokenizer).  Prints one JSON object per
-request ({"prompt_tokens", "token_ids", "text"}) and a last line with tokens per second.  A ragged family (Lokizen, Vumalix, Bamanex) runs prompt
+request ({"prompt_tokens", "token_ids", "text"}) and a last line with tokens per second.  A ragged family (Lokizen, Vumalix, Bamanex, Mikipel) runs prompt
 portions and decoded tokens of different requests in one batch per step; ``--max-num-batched-tokens`` is the step's budget and
 ``--page`` the size of a cache page."""
 from __future__ import annotations

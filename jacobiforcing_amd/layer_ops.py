@@ -596,12 +596,14 @@ def _addends(addends, n: int, W: int, what: str):
 
 def depth_mix_norm(x_in: torch.Tensor, addends: Sequence[Tuple[torch.Tensor, Optional[torch.Tensor]]], mult: float, streams: Optional[torch.Tensor],
                    depth: int, mix: Optional[torch.Tensor], x_out: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float,
-                   out_dtype: Optional[torch.dtype], want_float: bool = False):
+                   out_dtype: Optional[torch.dtype], want_float: bool = False, shift: Optional[tuple] = None):
     """Residual update, weighted sum over the streams of all depths, RMS norm.  y = x_in + mult * sum of the addends ((tensor [N, W] or
     [N, S, W], channel scale or None), at most three).  With ``depth`` >= 0, y becomes streams[depth] (``streams`` float [depths, N, W]) and
     x_out = sum_{j <= depth} mix[j] * streams[j] (``mix`` float, at least depth + 1 entries; None: x_out = y); with ``depth`` < 0, x_out = y,
     or nothing is written when there are no addends.  Returns the norm of x_out (of x_in when nothing was written) times ``w`` (float
-    [W] or None) in ``out_dtype`` — and, with ``want_float``, the same unrounded in float as a second result; None with neither."""
+    [W] or None) in ``out_dtype`` — and, with ``want_float``, the same unrounded in float as a second result; None with neither.
+    ``shift`` = (mu float [W], batch, tail float [slots, 1, W]): for a step in which every request brings ONE row, ``token_shift`` of the
+    unrounded norm in the same launch; its result (``out_dtype``) is appended to what is returned."""
     _dev(x_in)
     n, W = x_in.shape
     _need(x_in.dtype == torch.float32 and x_in.is_contiguous() and len(addends) <= 3, "depth_mix_norm: x_in contiguous float32 [N, W], at most 3 addends")
@@ -620,10 +622,21 @@ def depth_mix_norm(x_in: torch.Tensor, addends: Sequence[Tuple[torch.Tensor, Opt
         _need(w.dtype == torch.float32 and w.numel() == W and w.is_contiguous(), "depth_mix_norm: the norm weight is float [W]")
     out = torch.empty((n, W), dtype=out_dtype, device=x_in.device) if out_dtype is not None else None
     outf = torch.empty((n, W), dtype=torch.float32, device=x_in.device) if want_float else None
+    mu = seq = tail = outs = None
+    if shift is not None:
+        mu, batch, tail = shift
+        _need(out_dtype is not None and batch.N == n and batch.B == n and max(batch.counts) == 1, "depth_mix_norm: the shift in this launch needs one row per request")
+        _need(mu.dtype == torch.float32 and mu.numel() == W and mu.is_contiguous() and tail.dtype == torch.float32 and tail.is_contiguous() and
+              tail.numel() == tail.shape[0] * W and batch.max_slot < tail.shape[0], "depth_mix_norm: mu float [W], tail float [slots, 1, W] with the batch's slots")
+        seq, outs = batch.seq, torch.empty((n, W), dtype=out_dtype, device=x_in.device)
     N.check_layers(N.layers().jl_depth_mix_norm(_ptr(x_in), arr, len(addends), float(mult), _ptr(streams) if depth >= 0 else None, ld, int(depth),
                                                _ptr(mix) if depth >= 0 else None, _ptr(x_out) if written else None, _ptr(w), float(eps), _ptr(out),
-                                               _code(out_dtype or torch.float32), _ptr(outf), n, W, _stream(x_in.device)), "jl_depth_mix_norm")
-    return (out, outf) if want_float else out
+                                               _code(out_dtype or torch.float32), _ptr(outf), n, W, _ptr(mu), _ptr(seq), _ptr(tail), _ptr(outs),
+                                               _stream(x_in.device)), "jl_depth_mix_norm")
+    res = (out, outf) if want_float else out
+    if shift is not None:
+        return (*res, outs) if want_float else (res, outs)
+    return res
 
 
 def token_shift(h: torch.Tensor, mu: torch.Tensor, batch: RaggedBatch, tail: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:

@@ -17,7 +17,7 @@ token shift, h_t + (h_(t-1) - h_t) * mu per channel; the previous token's h is p
 The forward runs one ragged batch (``layer_ops.RaggedBatch``): portions of prompts and single decoded tokens side by side, over
 ``engine.state_cache.PagedStateCache``.  Dense products are torch's (hipBLASLt / rocBLAS); everything else is a launch of
 ``libjf_layers.so`` / ``libjf_layers_seq.so``.  A layer's sublayer outputs are folded into the launch that stores its result, mixes
-the depths and forms the next layer's norm.  With float32 weights every product is a true 32-bit one."""
+the depths and forms the next layer's norm — and, in a step of single tokens, its token shift.  With float32 weights every product is a true 32-bit one."""
 from __future__ import annotations
 
 import json
@@ -337,20 +337,27 @@ class MikipelModel:
         pending: list = []                               # the previous layer's sublayer outputs, folded into the next norm's launch
         both = dt != torch.float32                       # a 16-bit norm for the products, the unrounded one for the shift and the router
 
-        def hand_on(li: int, norm_w: Optional[torch.Tensor], out_dtype, unrounded: bool = False):
-            """Layer li - 1's result becomes stream li, the mixture of streams 0 .. li the new x; returns its norm."""
+        def hand_on(li: int, norm_w: Optional[torch.Tensor], out_dtype, unrounded: bool = False, shift=None):
+            """Layer li - 1's result becomes stream li, the mixture of streams 0 .. li the new x; returns its norm (and, with ``shift``,
+            the shifted norm from the same launch)."""
             nonlocal x, pending
             if not pending:
-                return LO.depth_mix_norm(x, [], mult, None, -1, None, None, norm_w, eps, out_dtype, want_float=unrounded)
-            r = LO.depth_mix_norm(x, pending, mult, streams, li, w.layers[li - 1]["dwa"], mixed, norm_w, eps, out_dtype, want_float=unrounded)
+                return LO.depth_mix_norm(x, [], mult, None, -1, None, None, norm_w, eps, out_dtype, want_float=unrounded, shift=shift)
+            r = LO.depth_mix_norm(x, pending, mult, streams, li, w.layers[li - 1]["dwa"], mixed, norm_w, eps, out_dtype, want_float=unrounded, shift=shift)
             x, pending = mixed, []
             return r
 
+        single = max(batch.counts) == 1                  # every request brings one row (decoding): the shift rides in the norm's launch
+
         for li, L in enumerate(cfg.layers):
             lw = w.layers[li]
-            hs = hand_on(li, lw["norm1"], dt, unrounded=both)
-            h, hf = hs if both else (hs, hs)
-            shifted = LO.token_shift(hf, lw["shift"], batch, cache.tails[li]["shift"], dt)
+            if single:
+                hs = hand_on(li, lw["norm1"], dt, unrounded=both, shift=(lw["shift"], batch, cache.tails[li]["shift"]))
+                h, hf, shifted = hs if both else (hs[0], hs[0], hs[1])
+            else:
+                hs = hand_on(li, lw["norm1"], dt, unrounded=both)
+                h, hf = hs if both else (hs, hs)
+                shifted = LO.token_shift(hf, lw["shift"], batch, cache.tails[li]["shift"], dt)
             mixer = self._attention if L["type"] == "attention" else self._latent_attention if L["type"] == "latent_attention" else self._delta
             pending = [(F.linear(mixer(li, shifted, batch, cache), lw["w_o"]), None)]
             if L.get("mlp") is not None:

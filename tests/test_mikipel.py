@@ -298,6 +298,18 @@ def test_token_shift_kernel_reads_and_moves_the_tail():
         prev = torch.stack([torch.zeros(W), h[0], h[1], tail[0, 0], tail[3, 0], h[4], torch.zeros(W)])         # a start at position 0 never reads its slot
         assert rel_err(out, h.double() + (prev.double() - h.double()) * mu.double()) < tol
         assert torch.equal(td.cpu()[:, 0], torch.stack([h[3], h[6], h[2], h[5]]))
+    # a step of single rows: the norm's launch shifts as well (the unrounded norm against the slot's tail, which it then replaces)
+    x, w = torch.randn(4, W, generator=g), torch.randn(W, generator=g)
+    b1 = LO.RaggedBatch.build([1, 1, 1, 1], [4, 0, 9, 1], [3, 1, 0, 2], [[0], [1], [2, 3], [4]], 8, "cuda")
+    hn = O.rms_norm(x.double(), w.double(), 1e-5)
+    prev = torch.stack([tail[3, 0], torch.zeros(W), tail[0, 0], tail[2, 0]]).double()
+    for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 6e-3)):
+        td.copy_(tail)
+        o16, o32, sh = LO.depth_mix_norm(x.cuda(), [], 1.0, None, -1, None, None, w.cuda(), 1e-5, dtype, want_float=True, shift=(mu.cuda(), b1, td))
+        assert rel_err(sh.float().cpu(), hn + (prev - hn) * mu.double()) < tol and rel_err(o32.cpu(), hn) < 1e-6 and o16.dtype == dtype
+        assert rel_err(td.cpu()[[3, 1, 0, 2], 0], hn) < 1e-6
+    with pytest.raises(ValueError):
+        LO.depth_mix_norm(h.cuda(), [], 1.0, None, -1, None, None, None, 1e-5, torch.float32, shift=(mu.cuda(), b, td))       # a request with three rows
 
 
 @gpu
