@@ -300,6 +300,106 @@ __global__ __launch_bounds__(256) void depth_mix_norm_kernel(const float *__rest
     }
 }
 
+// The same for widths in multiples of four with 16-byte aligned rows: a thread owns four consecutive channels per pass (16-byte loads and
+// stores of floats, 8-byte ones of bfloat16).  SHIFT: the token shift of single-row steps rides along.
+__device__ __forceinline__ void ld4_any(const void *p, int dtype, int64_t i, float (&v)[4]) {
+    if (dtype == JL_BF16) {
+        const uint2 t = *(const uint2 *)((const bf16_t *)p + i);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u); v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    } else {
+        const float4 t = *(const float4 *)((const float *)p + i);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+}
+__device__ __forceinline__ void st4_f(float *p, const float (&v)[4]) { *(float4 *)p = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void st4_f(bf16_t *p, const float (&v)[4]) {
+    bf16_t h[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st_f(&h[i], v[i]);
+    *(uint2 *)p = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+}
+
+template <typename T, bool SHIFT>
+__global__ __launch_bounds__(256) void depth_mix_norm_vec_kernel(const float *__restrict__ x_in, jl_addend a0, jl_addend a1, jl_addend a2, float mult,
+                                                                  float *__restrict__ streams, int64_t stream_ld, int depth, const float *__restrict__ mix,
+                                                                  float *__restrict__ x_out, const float *__restrict__ w, float eps, T *__restrict__ out,
+                                                                  float *__restrict__ out_f32, int W, const float *__restrict__ shift_mu,
+                                                                  const int32_t *__restrict__ seq, float *shift_tail, T *__restrict__ out_shift) {
+    __shared__ float red[16];
+    const int64_t n = blockIdx.x;
+    const jl_addend ad[3] = {a0, a1, a2};
+    const bool update = a0.y || a1.y || a2.y || depth >= 0;
+    float ss = 0.f;
+    for (int c = threadIdx.x * 4; c < W; c += 1024) {
+        float t[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            if (!ad[k].y) continue;
+            float u[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int s2 = 0; s2 < ad[k].count; ++s2) {
+                float a[4];
+                ld4_any(ad[k].y, ad[k].dtype, (n * ad[k].count + s2) * (int64_t)W + c, a);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) u[i] += a[i];
+            }
+            if (ad[k].scale) {
+                const float4 sc = *(const float4 *)(ad[k].scale + c);
+                u[0] *= sc.x; u[1] *= sc.y; u[2] *= sc.z; u[3] *= sc.w;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) t[i] += u[i];
+        }
+        float v[4];
+        ld4_any(x_in, JL_F32, n * W + c, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += mult * t[i];
+        if (depth >= 0) {
+            st4_f(streams + depth * stream_ld + n * W + c, v);
+            if (mix) {
+                const float md = mix[depth];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) v[i] *= md;
+                for (int j = 0; j < depth; ++j) {
+                    float sj[4];
+                    ld4_any(streams, JL_F32, j * stream_ld + n * W + c, sj);
+                    const float mj = mix[j];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] += mj * sj[i];
+                }
+            }
+        }
+        if (update) st4_f(x_out + n * W + c, v);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss += v[i] * v[i];
+    }
+    if (!out && !out_f32 && !SHIFT) return;
+    ss = block_sum_f32(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)W + eps);
+    const float *xr = update ? x_out + n * W : x_in + n * W;
+    int slot = 0;
+    bool past = false;
+    if (SHIFT) { slot = seq[4 * n + 3]; past = seq[4 * n + 2] > 0; }
+    for (int c = threadIdx.x * 4; c < W; c += 1024) {
+        float v[4], wv[4] = {1.f, 1.f, 1.f, 1.f};
+        ld4_any(xr, JL_F32, c, v);
+        if (w) ld4_any(w, JL_F32, c, wv);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= r * wv[i];
+        if (out) st4_f(out + n * W + c, v);
+        if (out_f32) st4_f(out_f32 + n * W + c, v);
+        if (SHIFT) {
+            float *tl = shift_tail + (int64_t)slot * W + c;
+            float prev[4] = {0.f, 0.f, 0.f, 0.f}, mu[4], sh[4];
+            if (past) ld4_any(tl, JL_F32, 0, prev);
+            st4_f(tl, v);
+            ld4_any(shift_mu, JL_F32, c, mu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sh[i] = v[i] + (prev[i] - v[i]) * mu[i];
+            st4_f(out_shift + n * W + c, sh);
+        }
+    }
+}
+
 extern "C" int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, int32_t n_addends, float mult, float *streams, int64_t stream_ld,
                                  int32_t depth, const float *mix, float *x_out, const float *w, float eps, void *out, int dtype, float *out_f32,
                                  int64_t N, int32_t W, const float *shift_mu, const int32_t *seq, float *shift_tail, void *out_shift, void *stream) {
@@ -316,9 +416,17 @@ extern "C" int jl_depth_mix_norm(const float *x_in, const jl_addend *addends, in
         ad[k] = addends[k];
         if (ad[k].y && ad[k].count <= 0) return jl_fail(JL_E_INVALID, "jl_depth_mix_norm: addend %d has no rows", k);
     }
-    JL_DISPATCH(dtype, depth_mix_norm_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x_in, ad[0], ad[1], ad[2], mult, streams, stream_ld, depth,
-                                                                                                    mix, x_out, w, eps, (T *)out, out_f32, W, shift_mu, seq,
-                                                                                                    shift_tail, (T *)out_shift));
+    // every pointer the four-channel form touches starts at a 16-byte border (8 for bfloat16 rows) and every row is a multiple of four wide
+    auto al = [](const void *q, uintptr_t a) { return ((uintptr_t)q % a) == 0; };
+    bool vec = W % 4 == 0 && stream_ld % 4 == 0 && al(x_in, 16) && al(x_out, 16) && al(streams, 16) && al(w, 16) && al(out_f32, 16) && al(shift_mu, 16) &&
+               al(shift_tail, 16) && al(out, dtype == JL_BF16 ? 8 : 16) && al(out_shift, dtype == JL_BF16 ? 8 : 16);
+    for (int k = 0; k < n_addends; ++k) vec = vec && al(ad[k].y, ad[k].dtype == JL_BF16 ? 8 : 16) && al(ad[k].scale, 16);
+    hipStream_t st = (hipStream_t)stream;
+#define DMN_ARGS x_in, ad[0], ad[1], ad[2], mult, streams, stream_ld, depth, mix, x_out, w, eps, (T *)out, out_f32, W, shift_mu, seq, shift_tail, (T *)out_shift
+    if (vec && shift_mu) JL_DISPATCH(dtype, (depth_mix_norm_vec_kernel<T, true><<<dim3((unsigned)N), 256, 0, st>>>(DMN_ARGS)));
+    else if (vec) JL_DISPATCH(dtype, (depth_mix_norm_vec_kernel<T, false><<<dim3((unsigned)N), 256, 0, st>>>(DMN_ARGS)));
+    else JL_DISPATCH(dtype, depth_mix_norm_kernel<T><<<dim3((unsigned)N), 256, 0, st>>>(DMN_ARGS));
+#undef DMN_ARGS
     return jl_check_launch("depth_mix_norm_kernel");
 }
 

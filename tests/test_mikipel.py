@@ -253,7 +253,7 @@ class Rig:
 
 
 @gpu
-@pytest.mark.parametrize("W", [96, 200, 1000])
+@pytest.mark.parametrize("W", [50, 96, 200, 1000, 2052])
 def test_residual_sum_depth_mixture_and_norm(W):
     from jacobiforcing_amd import layer_ops as LO
     g = torch.Generator().manual_seed(W)
