@@ -27,19 +27,19 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(const T *__restrict__ 
     const int64_t n = blockIdx.x;
     const T *row = proj + n * ld;
     float sq = 0.f, sk = 0.f;
-    for (int c = threadIdx.x; c < Rq; c += 256) { const float v = ld_f(row + q_col + c); sq += v * v; }
-    for (int c = threadIdx.x; c < R; c += 256) { const float v = ld_f(row + kv_col + c); sk += v * v; }
-    for (int c = threadIdx.x; c < rd; c += 256) kr[c] = ld_f(row + kv_col + R + c);
+    for (int c = threadIdx.x; c < Rq; c += blockDim.x) { const float v = ld_f(row + q_col + c); sq += v * v; }
+    for (int c = threadIdx.x; c < R; c += blockDim.x) { const float v = ld_f(row + kv_col + c); sk += v * v; }
+    for (int c = threadIdx.x; c < rd; c += blockDim.x) kr[c] = ld_f(row + kv_col + R + c);
     sq = block_sum_f32(sq, red);
     sk = block_sum_f32(sk, red);                                // its barriers also publish kr
     const float rq = Rq > 0 ? 1.0f / sqrtf(sq / (float)Rq + eps) : 0.f, rk = 1.0f / sqrtf(sk / (float)R + eps);
-    for (int c = threadIdx.x; c < Rq; c += 256) st_f(cq_out + n * Rq + c, ld_f(row + q_col + c) * rq * ld_f(wq + c));
+    for (int c = threadIdx.x; c < Rq; c += blockDim.x) st_f(cq_out + n * Rq + c, ld_f(row + q_col + c) * rq * ld_f(wq + c));
     const int64_t sl = slot[n];
     if (sl < 0) return;
     T *dst = pool + sl * (int64_t)(R + rd);
-    for (int c = threadIdx.x; c < R; c += 256) st_f(dst + c, ld_f(row + kv_col + c) * rk * ld_f(wkv + c));
+    for (int c = threadIdx.x; c < R; c += blockDim.x) st_f(dst + c, ld_f(row + kv_col + c) * rk * ld_f(wkv + c));
     const float *cs = cos_t + (int64_t)pos[n] * (rot_dims >> 1), *sn = sin_t + (int64_t)pos[n] * (rot_dims >> 1);
-    for (int c = threadIdx.x; c < rd; c += 256) st_f(dst + R + c, rot_half(kr, c, rot_dims, cs, sn, pairing));
+    for (int c = threadIdx.x; c < rd; c += blockDim.x) st_f(dst + R + c, rot_half(kr, c, rot_dims, cs, sn, pairing));
 }
 
 extern "C" int jl_latent_prep(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t Rq, int32_t kv_col, int32_t R,
@@ -53,7 +53,9 @@ extern "C" int jl_latent_prep(const void *proj, int dtype, int64_t N, int64_t ld
         return jl_fail(JL_E_INVALID, "jl_latent_prep: columns do not fit the row stride");
     if (rot_dims < 0 || rot_dims > rd || (rot_dims & 1) || (rot_dims && (!cos_t || !sin_t || table_len <= 0)))
         return jl_fail(JL_E_INVALID, "jl_latent_prep: rot_dims must be even, at most rd, with angle tables");
-    JL_DISPATCH(dtype, latent_prep_kernel<T><<<dim3((unsigned)N), 256, (size_t)(rd > 0 ? rd : 1) * 4, (hipStream_t)stream>>>(
+    // narrow rows (a few hundred values per token): one wavefront per token instead of four, of which three would idle
+    const int threads = (int64_t)Rq + R + rd <= 512 ? 64 : 256;
+    JL_DISPATCH(dtype, latent_prep_kernel<T><<<dim3((unsigned)N), threads, (size_t)(rd > 0 ? rd : 1) * 4, (hipStream_t)stream>>>(
                            (const T *)proj, ld, q_col, Rq, kv_col, R, rd, rot_dims, (const T *)wq, (const T *)wkv, eps, pos, cos_t, sin_t,
                            (T *)cq_out, (T *)pool, slot, pairing));
     return jl_check_launch("latent_prep_kernel");
