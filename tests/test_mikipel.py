@@ -5,7 +5,6 @@ and inputs are chosen so that it shows.
 
 CPU tests cover the oracle's own pieces, the config reader and the cache layout; everything that launches a kernel is marked ``gpu``."""
 import json
-import math
 import random
 
 import numpy as np
