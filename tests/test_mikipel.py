@@ -712,6 +712,28 @@ def test_greedy_generation_through_the_engine_and_its_scheduler(tmp_path):
 
 
 @gpu
+def test_a_preempted_request_starts_again_from_an_empty_state(tmp_path):
+    """Three pages for two requests that need five: the newer one is preempted while it decodes, gives pages and slot back and is
+    prefilled again later — its recurrent state, convolution inputs and shifted rows start from nothing, the results are the oracle's."""
+    from jacobiforcing_amd import LLM, SamplingParams
+    cfg_dict = shape_a()
+    tensors = tensors_for(cfg_dict, 43)
+    path = _write_model(tmp_path, cfg_dict, tensors)
+    V = cfg_dict["vocab"]
+    prompts = [toks(100, V, 61), toks(60, V, 62)]
+    llm = LLM(path, tokenizer_path="none", dtype="float32", kvcache_block_size=64, num_kvcache_blocks=3, max_num_seqs=2, max_model_len=192,
+              max_num_batched_tokens=192, device="cuda")
+    preempted = []
+    keep = llm.scheduler.preempt
+    llm.scheduler.preempt = lambda seq: (preempted.append(seq.seq_id), keep(seq))[1]
+    out = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=30, ignore_eos=True), use_tqdm=False)
+    assert preempted, "the pool was meant to run out"
+    for p, o in zip(prompts, out):
+        assert o["token_ids"] == _oracle_greedy(cfg_dict, tensors, p, 30)
+    assert len(llm.scheduler.block_manager.free_block_ids) == 3 and len(llm.model_runner.free_rows) == 2
+
+
+@gpu
 def test_sampling_through_the_engine_follows_the_distribution(tmp_path):
     from jacobiforcing_amd import LLM, SamplingParams
     cfg_dict = shape_b()
